@@ -1,0 +1,452 @@
+"""CPU oracle for the DFlash speculative-verify hot path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the shipped package may import this
+module: it is the checker the HIP kernels are compared against, used by
+``tests/``, by ``__graft_entry__.smoke()`` and by the ``cpu_baseline`` leg of
+``bench.py``.  It is a plain numpy restatement of the reference's *ops*
+implementations (the code SwiftLM runs when the default device is the CPU or
+``DFLASH_FORCE_OPS`` is set) and of the host-side accept / commit / rollback
+indexing.  Each function cites the reference lines it follows.
+
+The arithmetic underneath the reference's ops path lives in MLX (SharpAI/mlx via
+SharpAI/mlx-swift, a path dependency of Package.swift:16 whose version is not
+pinned and whose sources are absent from the reference tree).  MLX's own
+reduction order and rounding points are therefore not reproduced bit for bit;
+the functions below compute in a caller-chosen dtype (float32 mirrors the ops
+path after type promotion, float64 gives a ground truth for tolerance checks).
+
+Pinning status (what fixes each function other than its own formula):
+
+* ``tape_replay_ops``            closed form for scalar gates, prefix
+                                 composition, identities, fp64 brute force.
+* ``gated_delta_ops_with_tape``  textbook delta rule in matrix form
+                                 ``S <- g S (I - b k k^T) + b v k^T``, the
+                                 in-tree second restatement
+                                 (Sources/SwiftLM/KimiLinearDFlash.swift:383-405),
+                                 forward/replay consistency, special cases.
+* masked variants                equal the unmasked function on the sub-sequence
+                                 of unmasked steps.
+* ``match_acceptance_length``    the reference's own documented example
+                                 (DFlashRuntime.swift:130-132) + brute force.
+* ``rebuild_conv_state``, ``restore_target_cache_after_acceptance``,
+  ``accept_commit``              integer indexing, brute force.
+* ``sdpa_block_causal``          library softmax / logsumexp (scipy), row-sum
+                                 invariants, reduction to plain causal attention.
+* ``sdpa_2pass``                 must agree with ``sdpa_block_causal``.
+
+The reference holds no golden vectors for any of these (its only numeric check
+is Metal-vs-ops ``cos > 0.999 and max_abs_diff < 0.01``,
+tests/DFlash/DFlashProfiler.swift:215-244), so the bit-level behaviour of MLX on
+this path is "parity unpinned"; everything is held to the stated tolerances.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+# ----------------------------------------------------------------------------
+# bf16 / f16 helpers (numpy has no bfloat16)
+# ----------------------------------------------------------------------------
+
+
+def round_to_bf16(x: np.ndarray) -> np.ndarray:
+    """Round float32 values to the nearest bfloat16 (ties to even); returns float32."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32).astype(np.uint64)
+    nan = np.isnan(x)
+    rounded = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    out = rounded.astype(np.uint32).view(np.float32).copy()
+    out[nan] = np.nan
+    return out.reshape(x.shape)
+
+
+def round_to_f16(x: np.ndarray) -> np.ndarray:
+    return np.asarray(x, dtype=np.float32).astype(np.float16).astype(np.float32)
+
+
+def quantize(x: np.ndarray, dtype: str | None) -> np.ndarray:
+    """Round to ``dtype`` ('f32' | 'bf16' | 'f16' | None) and return in x's dtype."""
+    if dtype in (None, "f32", "f64"):
+        return x
+    if dtype == "bf16":
+        return round_to_bf16(x.astype(np.float32)).astype(x.dtype)
+    if dtype == "f16":
+        return round_to_f16(x.astype(np.float32)).astype(x.dtype)
+    raise ValueError(dtype)
+
+
+# ----------------------------------------------------------------------------
+# a1  tape replay
+# ----------------------------------------------------------------------------
+
+
+def _repeat_heads(x: np.ndarray, rf: int) -> np.ndarray:
+    # MLX.repeated(k, count: rf, axis: 2): consecutive repeat, value head hv
+    # reads key head hv // rf (DFlashKernels.swift:384 and :47).
+    return np.repeat(x, rf, axis=2) if rf > 1 else x
+
+
+def tape_replay_ops(tape, k, g, state, mask=None, *, dtype=np.float32, requant=None):
+    """Replay an innovation tape through the recurrent state.
+
+    Follows ``tapeReplayOps`` (Sources/DFlash/DFlashKernels.swift:371-407):
+    for each step ``state = state * decay + delta * k``, with ``decay`` the
+    multiplicative gate (scalar per head ``[B,T,Hv]`` or per channel
+    ``[B,T,Hv,Dk]``), and a masked step leaving the state untouched
+    (``MLX.where(stepMask, state, prev)``, :399-403).
+
+    ``requant`` ('bf16' | 'f16') re-rounds the state after every step, which
+    is what the Metal kernel does for a low-precision state
+    (DFlashKernels.swift:70); None follows the ops path.
+
+    Shapes: tape [B,T,Hv,Dv], k [B,T,Hk,Dk], state [B,Hv,Dv,Dk], mask [B,T].
+    """
+    tape = np.asarray(tape, dtype=dtype)
+    k = np.asarray(k, dtype=dtype)
+    g = np.asarray(g, dtype=dtype)
+    state = np.asarray(state, dtype=dtype).copy()
+    T = tape.shape[1]
+    Hk, Hv = k.shape[2], tape.shape[2]
+    k = _repeat_heads(k, Hv // Hk)
+    for t in range(T):
+        prev = state
+        if g.ndim == 4:
+            decay = g[:, t, :, None, :]
+        else:
+            decay = g[:, t, :, None, None]
+        delta = tape[:, t, :, :, None]
+        kT = k[:, t, :, None, :]
+        state = quantize(state * decay + delta * kT, requant)
+        if mask is not None:
+            step = (np.asarray(mask)[:, t] > 0.5)[:, None, None, None]
+            state = np.where(step, state, prev)
+    return state
+
+
+# ----------------------------------------------------------------------------
+# a2  gated delta forward with tape
+# ----------------------------------------------------------------------------
+
+
+def gated_delta_ops_with_tape(q, k, v, g, beta, state, mask=None, *, dtype=np.float32,
+                              requant=None):
+    """GatedDelta forward that also records the innovation tape.
+
+    Follows ``gatedDeltaOpsWithTape`` (DFlashKernels.swift:409-466): per step
+    ``S' = S*decay``; ``kv_mem = sum_dk S'*k``; ``delta = (v - kv_mem)*beta``;
+    ``S = S' + k (x) delta``; ``y = sum_dk S*q``.  A masked step keeps S and
+    emits y = 0 and delta = 0 (:446-453).
+
+    Returns (y [B,T,Hv,Dv], state [B,Hv,Dv,Dk], tape [B,T,Hv,Dv] float32).
+    """
+    q = np.asarray(q, dtype=dtype)
+    k = np.asarray(k, dtype=dtype)
+    v = np.asarray(v, dtype=dtype)
+    g = np.asarray(g, dtype=dtype)
+    beta = np.asarray(beta, dtype=dtype)
+    state = np.asarray(state, dtype=dtype).copy()
+    B, T, Hk, Dk = q.shape
+    Hv = v.shape[2]
+    q = _repeat_heads(q, Hv // Hk)
+    k = _repeat_heads(k, Hv // Hk)
+    ys, tapes = [], []
+    for t in range(T):
+        if g.ndim == 4:
+            decay = g[:, t, :, None, :]
+        else:
+            decay = g[:, t, :, None, None]
+        decayed = state * decay
+        kt = k[:, t, :, None, :]
+        kv_mem = (decayed * kt).sum(axis=-1)
+        delta = (v[:, t] - kv_mem) * beta[:, t, :, None]
+        new_state = quantize(decayed + kt * delta[..., None], requant)
+        y = (new_state * q[:, t, :, None, :]).sum(axis=-1)
+        if mask is not None:
+            step = np.asarray(mask)[:, t] > 0.5
+            sg = step[:, None, None, None]
+            yg = step[:, None, None]
+            state = np.where(sg, new_state, state)
+            ys.append(np.where(yg, y, 0))
+            tapes.append(np.where(yg, delta, 0))
+        else:
+            state = new_state
+            ys.append(y)
+            tapes.append(delta)
+    y = np.stack(ys, axis=1)
+    tape = np.stack(tapes, axis=1)
+    if dtype == np.float32:
+        tape = tape.astype(np.float32)
+    return y, state, tape
+
+
+# ----------------------------------------------------------------------------
+# a5 / a6  acceptance length and commit indexing
+# ----------------------------------------------------------------------------
+
+
+def match_acceptance_length(drafted, posterior) -> int:
+    """Number of leading positions where drafted == posterior.
+
+    ``sum(cumprod(drafted == posterior))``; empty input gives 0
+    (Sources/DFlash/DFlashRuntime.swift:133-142).
+    """
+    drafted = np.asarray(drafted).reshape(-1)
+    posterior = np.asarray(posterior).reshape(-1)
+    if drafted.shape[0] == 0:
+        return 0
+    matches = (drafted == posterior[: drafted.shape[0]]).astype(np.int32)
+    return int(np.cumprod(matches).sum())
+
+
+def accept_commit(staged_first: int, drafted, posterior, start: int):
+    """One verify cycle's integer bookkeeping (DFlashRuntime.swift:484-581).
+
+    ``drafted`` are the block's draft tokens *after* the staged first token
+    (length V-1); ``posterior`` the target's greedy tokens for all V verify
+    positions.  Returns a dict with the reference's names.
+    """
+    drafted = np.asarray(drafted).reshape(-1)
+    posterior = np.asarray(posterior).reshape(-1)
+    verify_ids = np.concatenate([[staged_first], drafted]).astype(np.int64)   # :490-493
+    V = verify_ids.shape[0]
+    if V > 1:
+        acceptance_len = match_acceptance_length(verify_ids[1:], posterior[: V - 1])  # :525-530
+    else:
+        acceptance_len = 0
+    commit_count = 1 + acceptance_len                                          # :544
+    committed = verify_ids[:commit_count]                                      # :545
+    staged_next = int(posterior[acceptance_len])                               # :547
+    new_start = start + commit_count                                           # :571
+    return {
+        "acceptance_len": acceptance_len,
+        "commit_count": commit_count,
+        "committed": committed,
+        "staged_next": staged_next,
+        "start": new_start,
+        # arguments handed to engine.rollback (:573-578)
+        "rollback_args": {"target_len": new_start, "acceptance_length": acceptance_len,
+                          "drafted_tokens": V - 1},
+    }
+
+
+# ----------------------------------------------------------------------------
+# a3  rollback cache
+# ----------------------------------------------------------------------------
+
+
+def rebuild_conv_state(snapshot_conv, tape_qkv, accepted_steps: int, keep: int = 3):
+    """Conv window after accepting ``accepted_steps`` tokens.
+
+    ``concat([snapshot_conv, tape_qkv], axis=1)[:, s : min(s + keep, len)]``
+    with ``s = accepted_steps`` (RecurrentRollbackCache.swift:139-158).  A
+    missing snapshot counts as ``keep`` rows of zeros (:147-152).
+    """
+    tape_qkv = np.asarray(tape_qkv)
+    if keep <= 0:
+        return None
+    if snapshot_conv is None:
+        snapshot_conv = np.zeros((tape_qkv.shape[0], keep, tape_qkv.shape[-1]), tape_qkv.dtype)
+    conv_input = np.concatenate([np.asarray(snapshot_conv), tape_qkv], axis=1)
+    start = accepted_steps
+    end = min(start + keep, conv_input.shape[1])
+    return conv_input[:, start:end]
+
+
+class RecurrentRollbackCacheOracle:
+    """State machine of ``RecurrentRollbackCache`` (RecurrentRollbackCache.swift:34-182)."""
+
+    def __init__(self, conv_kernel_size: int = 4):
+        self.keep = conv_kernel_size - 1
+        self.slots = [None, None]          # [conv state, recurrent state]
+        self.offset = 0
+        self.armed = False
+        self._tape = self._k = self._g = self._qkv = None
+        self._snapshot = None
+
+    def arm_rollback(self, prefix_len: int = 0):            # :63-71
+        self.armed = True
+        self._tape = self._k = self._g = self._qkv = None
+        self._snapshot = [self.slots[0], self.slots[1]]
+
+    def record_tape(self, tape, k, g, qkv):                 # :75-85
+        self._tape, self._k, self._g, self._qkv = tape, k, g, qkv
+
+    def rollback(self, n_accepted: int, *, dtype=np.float32):  # :95-131
+        if self._snapshot is None:
+            self.clear_transients()
+            return
+        snap = self._snapshot
+        if snap[0] is not None:
+            self.slots[0] = snap[0]
+        if snap[1] is not None:
+            self.slots[1] = snap[1]
+        if self._tape is not None and self._k is not None and self._g is not None \
+                and self.slots[1] is not None:
+            steps = n_accepted + 1                           # :115
+            self.slots[1] = tape_replay_ops(self._tape[:, :steps], self._k[:, :steps],
+                                            self._g[:, :steps], self.slots[1], dtype=dtype)
+            if self._qkv is not None:
+                self.slots[0] = rebuild_conv_state(snap[0], self._qkv, steps, self.keep)
+        self.clear_transients()
+
+    def clear_transients(self):                              # :163-170
+        self.armed = False
+        self._tape = self._k = self._g = self._qkv = None
+        self._snapshot = None
+
+    def trim(self, n: int) -> int:                           # :175-181
+        trimmed = min(self.offset, n)
+        self.offset -= trimmed
+        return trimmed
+
+
+def restore_target_cache_after_acceptance(caches, target_len, acceptance_length, drafted_tokens):
+    """Per-cache action list of ``restoreTargetCacheAfterAcceptance``.
+
+    (Sources/DFlash/DFlashRuntime.swift:188-223.)  ``caches`` is a list of
+    ``(kind, offset)`` with kind in {'rollback', 'mamba', 'kv'}; returns, per
+    cache, one of ('clear',), ('rollback', n_accepted), ('set_offset', n),
+    ('trim', n), ('none',).
+    """
+    fully = drafted_tokens > 0 and acceptance_length == drafted_tokens
+    out = []
+    for kind, offset in caches:
+        if kind == "rollback":
+            out.append(("clear",) if fully else ("rollback", acceptance_length))
+        elif kind == "mamba":
+            out.append(("set_offset", target_len))
+        elif kind == "kv":
+            out.append(("trim", offset - target_len) if offset > target_len else ("none",))
+        else:
+            raise ValueError(kind)
+    return out
+
+
+# ----------------------------------------------------------------------------
+# a8  block-causal GQA SDPA
+# ----------------------------------------------------------------------------
+
+
+def sdpa_block_causal(q, k, v, scale, mask=None, *, dtype=np.float64):
+    """``softmax(scale * Q K^T + causal [+ mask]) V`` for a draft block.
+
+    Q [B,Hq,M,D]; K,V [B,Hk,N,D] where N already includes the M block tokens;
+    row i sees keys ``0 .. N-M+i`` (DFlashKernels.swift:614).  GQA head mapping
+    ``hk = hq // (Hq/Hk)`` (:575).  ``mask`` is an optional additive
+    [B,Hq,M,N] (:548-553).  Returns (O [B,Hq,M,D], lse [B,Hq,M]) in ``dtype``;
+    ``lse = max + log(sum exp)`` of the scaled, masked scores (natural log).
+
+    This is what ``sdpaFallback`` (:818-828) asks of
+    MLXFast.scaledDotProductAttention when handed the same causal mask.
+    """
+    q = np.asarray(q, dtype=dtype)
+    k = np.asarray(k, dtype=dtype)
+    v = np.asarray(v, dtype=dtype)
+    B, Hq, M, D = q.shape
+    Hk, N = k.shape[1], k.shape[2]
+    rf = Hq // Hk
+    out = np.empty((B, Hq, M, v.shape[3]), dtype=dtype)
+    lse = np.empty((B, Hq, M), dtype=dtype)
+    rows = np.arange(M)[:, None]
+    cols = np.arange(N)[None, :]
+    visible = cols <= (N - M + rows)
+    for b in range(B):
+        for h in range(Hq):
+            hk = h // rf
+            s = (q[b, h] * dtype(scale)) @ k[b, hk].T          # scale folded into Q (:594)
+            if mask is not None:
+                s = s + np.asarray(mask[b, h], dtype=dtype)
+            s = np.where(visible, s, -np.inf)
+            m = s.max(axis=-1, keepdims=True)
+            p = np.exp(s - m)
+            l = p.sum(axis=-1, keepdims=True)
+            out[b, h] = (p @ v[b, hk]) / l
+            lse[b, h] = (m + np.log(l))[:, 0]
+    return out, lse
+
+
+def sdpa_2pass(q, k, v, scale, blocks=32, *, partial_dtype="bf16"):
+    """Restatement of the reference's split-KV two-pass kernels in float32.
+
+    Pass 1 (DFlashKernels.swift:563-649): block ``b`` of ``blocks`` walks keys
+    ``b, b+blocks, ...`` with an online softmax and stores an unnormalised
+    partial O rounded to the input type (:647) plus fp32 max / sum.
+    Pass 2 (:661-720): global max, rescaled sum, weighted partial sum, divide
+    unless the sum is 0.  Returns O float32 [B,Hq,M,D] (before the final cast).
+    """
+    q = np.asarray(q, dtype=np.float32)
+    k = np.asarray(k, dtype=np.float32)
+    v = np.asarray(v, dtype=np.float32)
+    B, Hq, M, D = q.shape
+    Hk, N = k.shape[1], k.shape[2]
+    rf = Hq // Hk
+    fmin = np.finfo(np.float32).min
+    out = np.zeros((B, Hq, M, D), np.float32)
+    for b in range(B):
+        for h in range(Hq):
+            hk = h // rf
+            qs = np.float32(scale) * q[b, h]
+            part = np.zeros((M, blocks, D), np.float32)
+            sums = np.zeros((M, blocks), np.float32)
+            maxs = np.full((M, blocks), fmin, np.float32)
+            for blk in range(blocks):
+                idx = np.arange(blk, N, blocks)
+                if idx.size == 0:
+                    continue
+                s = qs @ k[b, hk, idx].T                               # [M, n_blk]
+                use = idx[None, :] <= (N - M + np.arange(M)[:, None])
+                s = np.where(use, s, -np.inf)
+                mx = np.maximum(s.max(axis=-1), fmin)
+                p = np.where(use, np.exp(s - mx[:, None]), 0).astype(np.float32)
+                sums[:, blk] = p.sum(axis=-1)
+                maxs[:, blk] = mx
+                part[:, blk] = quantize((p @ v[b, hk, idx]).astype(np.float32), partial_dtype)
+            gmax = maxs.max(axis=-1)
+            w = np.exp(maxs - gmax[:, None]).astype(np.float32)
+            tot = (w * sums).sum(axis=-1)
+            o = (w[:, :, None] * part).sum(axis=1)
+            out[b, h] = np.where(tot[:, None] == 0, o, o / np.where(tot == 0, 1, tot)[:, None])
+    return out
+
+
+# ----------------------------------------------------------------------------
+# synthetic inputs of the BASELINE configs
+# ----------------------------------------------------------------------------
+
+
+def _softplus(x):
+    return np.log1p(np.exp(-np.abs(x))) + np.maximum(x, 0)
+
+
+def make_gdn_inputs(seed, B, T, Hk, Hv, Dk, Dv, *, in_dtype="f32", vec_gate=False):
+    """q,k L2-normalised N(0,1); v N(0,1); beta sigmoid(N(0,1)); g = exp(-softplus(N(0,1)))
+    (the multiplicative decay the kernels take); state N(0, 0.1).  Inputs are rounded to
+    ``in_dtype`` and returned as float32; the state stays float32."""
+    rng = np.random.default_rng(seed)
+    q = rng.standard_normal((B, T, Hk, Dk)).astype(np.float32)
+    k = rng.standard_normal((B, T, Hk, Dk)).astype(np.float32)
+    q /= np.linalg.norm(q, axis=-1, keepdims=True)
+    k /= np.linalg.norm(k, axis=-1, keepdims=True)
+    v = rng.standard_normal((B, T, Hv, Dv)).astype(np.float32)
+    beta = (1.0 / (1.0 + np.exp(-rng.standard_normal((B, T, Hv))))).astype(np.float32)
+    gshape = (B, T, Hv, Dk) if vec_gate else (B, T, Hv)
+    g = np.exp(-_softplus(rng.standard_normal(gshape))).astype(np.float32)
+    state = (0.1 * rng.standard_normal((B, Hv, Dv, Dk))).astype(np.float32)
+    q, k, v, beta, g = (quantize(a, in_dtype) for a in (q, k, v, beta, g))
+    return dict(q=q, k=k, v=v, beta=beta, g=g, state=state)
+
+
+def draw_accepted(rng, T, kind="uniform"):
+    """BASELINE's accepted length n in [1, T]: uniform (config 0) or Geometric(0.25) clipped."""
+    if kind == "uniform":
+        return int(rng.integers(1, T + 1))
+    return int(min(rng.geometric(0.25), T))
+
+
+def make_sdpa_inputs(seed, B, Hq, Hk, M, L, D):
+    """bf16-rounded N(0,1) Q [B,Hq,M,D], K,V [B,Hk,L+M,D] as float32."""
+    rng = np.random.default_rng(seed)
+    q = round_to_bf16(rng.standard_normal((B, Hq, M, D)).astype(np.float32))
+    k = round_to_bf16(rng.standard_normal((B, Hk, L + M, D)).astype(np.float32))
+    v = round_to_bf16(rng.standard_normal((B, Hk, L + M, D)).astype(np.float32))
+    return q, k, v

@@ -1,0 +1,433 @@
+"""Pins the CPU oracle against what the mathematics fixes.
+
+The reference ships no golden vectors for this path, so every oracle function
+is checked against an independent formulation (closed forms, matrix form of the
+delta rule, library softmax/logsumexp, brute force), chosen so that a dropped
+term, a wrong sign or index, or a transposed operand fails at least one test.
+"""
+
+import numpy as np
+import pytest
+from scipy.special import logsumexp, softmax
+
+from oracle import dflash_oracle as O
+
+F64 = np.float64
+
+
+def _gdn(seed, B=2, T=6, Hk=2, Hv=4, Dk=8, Dv=5, vec=False):
+    d = O.make_gdn_inputs(seed, B, T, Hk, Hv, Dk, Dv, vec_gate=vec)
+    rng = np.random.default_rng(seed + 1000)
+    d["tape"] = rng.standard_normal((B, T, Hv, Dv)).astype(np.float32)
+    return d
+
+
+# ------------------------------------------------------------------ replay --
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_replay_scalar_gate_closed_form(seed):
+    d = _gdn(seed)
+    B, T, Hv, Dv = d["tape"].shape
+    Hk, Dk = d["k"].shape[2:]
+    got = O.tape_replay_ops(d["tape"], d["k"], d["g"], d["state"], dtype=F64)
+    g = d["g"].astype(F64)                                  # [B,T,Hv]
+    # suffix products  c_t = prod_{s>t} g_s
+    c = np.ones((B, T, Hv))
+    for t in range(T - 2, -1, -1):
+        c[:, t] = c[:, t + 1] * g[:, t + 1]
+    total = g.prod(axis=1)                                  # [B,Hv]
+    k_rep = np.repeat(d["k"].astype(F64), Hv // Hk, axis=2)  # [B,T,Hv,Dk]
+    want = total[:, :, None, None] * d["state"].astype(F64) + np.einsum(
+        "bth,bthv,bthk->bhvk", c, d["tape"].astype(F64), k_rep)
+    np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-14)
+
+
+def test_replay_vector_gate_closed_form():
+    d = _gdn(3, vec=True)
+    B, T, Hv, Dv = d["tape"].shape
+    Hk, Dk = d["k"].shape[2:]
+    got = O.tape_replay_ops(d["tape"], d["k"], d["g"], d["state"], dtype=F64)
+    g = d["g"].astype(F64)                                  # [B,T,Hv,Dk]
+    c = np.ones_like(g)
+    for t in range(T - 2, -1, -1):
+        c[:, t] = c[:, t + 1] * g[:, t + 1]
+    k_rep = np.repeat(d["k"].astype(F64), Hv // Hk, axis=2)
+    want = g.prod(axis=1)[:, :, None, :] * d["state"].astype(F64) + np.einsum(
+        "bthk,bthv,bthk->bhvk", c, d["tape"].astype(F64), k_rep)
+    np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-14)
+
+
+def test_replay_identities():
+    d = _gdn(4)
+    S0 = d["state"]
+    # zero steps
+    out = O.tape_replay_ops(d["tape"][:, :0], d["k"][:, :0], d["g"][:, :0], S0)
+    np.testing.assert_array_equal(out, S0)
+    # all-zero mask: untouched, not even decayed (DFlashKernels.swift:30-34)
+    mask = np.zeros(d["tape"].shape[:2], np.float32)
+    np.testing.assert_array_equal(O.tape_replay_ops(d["tape"], d["k"], d["g"], S0, mask), S0)
+    # delta = 0, g = 1
+    out = O.tape_replay_ops(np.zeros_like(d["tape"]), d["k"], np.ones_like(d["g"]), S0)
+    np.testing.assert_array_equal(out, S0)
+    # g = 0 on the last step: only the last outer product survives
+    g = d["g"].copy()
+    g[:, -1] = 0
+    out = O.tape_replay_ops(d["tape"], d["k"], g, S0, dtype=F64)
+    k_rep = np.repeat(d["k"], 2, axis=2).astype(F64)
+    want = d["tape"][:, -1, :, :, None].astype(F64) * k_rep[:, -1, :, None, :]
+    np.testing.assert_allclose(out, want, rtol=0, atol=1e-15)
+
+
+def test_replay_is_not_symmetric_in_dv_dk():
+    # state is [.., Dv, Dk]: delta indexes rows, k indexes columns.
+    d = _gdn(5, B=1, T=1, Hk=1, Hv=1, Dk=3, Dv=2)
+    tape = np.array([[[[1.0, 2.0]]]], np.float32)
+    k = np.array([[[[10.0, 20.0, 30.0]]]], np.float32)
+    out = O.tape_replay_ops(tape, k, np.zeros((1, 1, 1), np.float32), d["state"])
+    np.testing.assert_array_equal(out[0, 0], [[10, 20, 30], [20, 40, 60]])
+
+
+def test_replay_gqa_head_mapping_is_consecutive_repeat():
+    # value head hv reads key head hv // (Hv/Hk): heads 0,1 -> key head 0; 2,3 -> key head 1.
+    B, T, Hk, Hv, Dk, Dv = 1, 1, 2, 4, 4, 3
+    k = np.zeros((B, T, Hk, Dk), np.float32)
+    k[0, 0, 1] = 1.0                                     # only key head 1 is non-zero
+    tape = np.ones((B, T, Hv, Dv), np.float32)
+    out = O.tape_replay_ops(tape, k, np.ones((B, T, Hv), np.float32),
+                            np.zeros((B, Hv, Dv, Dk), np.float32))
+    assert np.all(out[0, :2] == 0) and np.all(out[0, 2:] == 1)
+
+
+@pytest.mark.parametrize("vec", [False, True])
+def test_replay_prefix_composition(vec):
+    d = _gdn(6, vec=vec)
+    full = O.tape_replay_ops(d["tape"], d["k"], d["g"], d["state"], dtype=F64)
+    for m in range(0, 7):
+        head = O.tape_replay_ops(d["tape"][:, :m], d["k"][:, :m], d["g"][:, :m], d["state"], dtype=F64)
+        both = O.tape_replay_ops(d["tape"][:, m:], d["k"][:, m:], d["g"][:, m:], head, dtype=F64)
+        np.testing.assert_allclose(both, full, rtol=1e-13, atol=1e-15)
+
+
+def test_replay_masked_equals_subsequence():
+    d = _gdn(7, B=1)
+    mask = np.array([[1, 0, 1, 1, 0, 1]], np.float32)
+    keep = mask[0] > 0.5
+    got = O.tape_replay_ops(d["tape"], d["k"], d["g"], d["state"], mask)
+    want = O.tape_replay_ops(d["tape"][:, keep], d["k"][:, keep], d["g"][:, keep], d["state"])
+    np.testing.assert_array_equal(got, want)
+
+
+def test_replay_requant_rounds_each_step():
+    d = _gdn(8, T=3)
+    out = O.tape_replay_ops(d["tape"], d["k"], d["g"], O.round_to_bf16(d["state"]), requant="bf16")
+    np.testing.assert_array_equal(out, O.round_to_bf16(out))
+    loose = O.tape_replay_ops(d["tape"], d["k"], d["g"], O.round_to_bf16(d["state"]))
+    assert not np.array_equal(out, loose)
+    np.testing.assert_allclose(out, loose, rtol=3e-2, atol=3e-2)
+
+
+# ------------------------------------------------------------- gated delta --
+
+
+def _matrix_form(q, k, v, g, beta, S0):
+    """Independent statement: S <- S diag(g) (I - b k k^T) + b v k^T per head, y = S q."""
+    B, T, Hk, Dk = q.shape
+    Hv, Dv = v.shape[2:]
+    rf = Hv // Hk
+    S = S0.astype(F64).copy()
+    ys = np.zeros((B, T, Hv, Dv))
+    deltas = np.zeros((B, T, Hv, Dv))
+    eye = np.eye(Dk)
+    for b in range(B):
+        for h in range(Hv):
+            M = S[b, h]                                   # [Dv, Dk]
+            for t in range(T):
+                kk = k[b, t, h // rf].astype(F64)
+                qq = q[b, t, h // rf].astype(F64)
+                gv = g[b, t, h].astype(F64)
+                G = np.diag(np.broadcast_to(gv, (Dk,)))
+                bt = F64(beta[b, t, h])
+                Md = M @ G
+                deltas[b, t, h] = bt * (v[b, t, h].astype(F64) - Md @ kk)
+                M = Md @ (eye - bt * np.outer(kk, kk)) + bt * np.outer(v[b, t, h].astype(F64), kk)
+                ys[b, t, h] = M @ qq
+            S[b, h] = M
+    return ys, S, deltas
+
+
+@pytest.mark.parametrize("vec", [False, True])
+def test_gated_delta_matches_matrix_form(vec):
+    d = _gdn(10, vec=vec)
+    y, S, tape = O.gated_delta_ops_with_tape(d["q"], d["k"], d["v"], d["g"], d["beta"], d["state"], dtype=F64)
+    yw, Sw, tw = _matrix_form(d["q"], d["k"], d["v"], d["g"], d["beta"], d["state"])
+    np.testing.assert_allclose(y, yw, rtol=1e-11, atol=1e-13)
+    np.testing.assert_allclose(S, Sw, rtol=1e-11, atol=1e-13)
+    np.testing.assert_allclose(tape, tw, rtol=1e-11, atol=1e-13)
+
+
+def test_gated_delta_matches_kimi_restatement():
+    # Second in-tree statement of the recurrence, vector gate, Hk == Hv
+    # (Sources/SwiftLM/KimiLinearDFlash.swift:395-403), written with einsum.
+    d = _gdn(11, Hk=4, Hv=4, vec=True)
+    q, k, v, g, beta = (d[n].astype(F64) for n in ("q", "k", "v", "g", "beta"))
+    s = d["state"].astype(F64)
+    ys = []
+    for t in range(q.shape[1]):
+        s = s * g[:, t][:, :, None, :]
+        kv = np.einsum("bhvk,bhk->bhv", s, k[:, t])
+        delta = (v[:, t] - kv) * beta[:, t][..., None]
+        s = s + np.einsum("bhk,bhv->bhvk", k[:, t], delta)
+        ys.append(np.einsum("bhvk,bhk->bhv", s, q[:, t]))
+    y, S, _ = O.gated_delta_ops_with_tape(d["q"], d["k"], d["v"], d["g"], d["beta"], d["state"], dtype=F64)
+    np.testing.assert_allclose(y, np.stack(ys, 1), rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(S, s, rtol=1e-12, atol=1e-14)
+
+
+@pytest.mark.parametrize("vec", [False, True])
+def test_forward_tape_replays_to_forward_state(vec):
+    """replay(tape[:n]) from S0 == state after the forward on the first n tokens."""
+    d = _gdn(12, vec=vec)
+    _, S_full, tape = O.gated_delta_ops_with_tape(d["q"], d["k"], d["v"], d["g"], d["beta"], d["state"], dtype=F64)
+    T = d["q"].shape[1]
+    for n in range(0, T + 1):
+        _, S_n, _ = O.gated_delta_ops_with_tape(d["q"][:, :n], d["k"][:, :n], d["v"][:, :n], d["g"][:, :n],
+                                                d["beta"][:, :n], d["state"], dtype=F64) if n else (0, d["state"].astype(F64), 0)
+        rep = O.tape_replay_ops(tape[:, :n], d["k"][:, :n], d["g"][:, :n], d["state"], dtype=F64)
+        np.testing.assert_allclose(rep, S_n, rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(O.tape_replay_ops(tape, d["k"], d["g"], d["state"], dtype=F64), S_full,
+                               rtol=1e-12, atol=1e-14)
+
+
+def test_gated_delta_special_cases():
+    d = _gdn(13, B=1, T=3, Hk=1, Hv=2, Dk=6, Dv=4)
+    # beta = 0: pure decay, delta = 0, y_t = decayed state . q_t
+    y, S, tape = O.gated_delta_ops_with_tape(d["q"], d["k"], d["v"], d["g"], np.zeros_like(d["beta"]),
+                                             d["state"], dtype=F64)
+    assert np.all(tape == 0)
+    dec = d["state"].astype(F64)
+    for t in range(3):
+        dec = dec * d["g"][:, t, :, None, None]
+        np.testing.assert_allclose(y[:, t], np.einsum("bhvk,bk->bhv", dec, d["q"][:, t, 0].astype(F64)),
+                                   rtol=1e-13)
+    np.testing.assert_allclose(S, dec, rtol=1e-13)
+    # zero state: the first innovation is beta * v and y_0 = beta * v * (k . q)
+    y, S, tape = O.gated_delta_ops_with_tape(d["q"], d["k"], d["v"], d["g"], d["beta"],
+                                             np.zeros_like(d["state"]), dtype=F64)
+    bv = d["beta"][:, 0, :, None].astype(F64) * d["v"][:, 0].astype(F64)
+    np.testing.assert_allclose(tape[:, 0], bv, rtol=1e-13)
+    kq = float(d["k"][0, 0, 0].astype(F64) @ d["q"][0, 0, 0].astype(F64))
+    np.testing.assert_allclose(y[:, 0], bv * kq, rtol=1e-12)
+
+
+@pytest.mark.parametrize("vec", [False, True])
+def test_gated_delta_masked_equals_subsequence(vec):
+    d = _gdn(14, B=1, vec=vec)
+    mask = np.array([[0, 1, 1, 0, 1, 0]], np.float32)
+    keep = mask[0] > 0.5
+    y, S, tape = O.gated_delta_ops_with_tape(d["q"], d["k"], d["v"], d["g"], d["beta"], d["state"], mask)
+    ys, Ss, ts = O.gated_delta_ops_with_tape(d["q"][:, keep], d["k"][:, keep], d["v"][:, keep], d["g"][:, keep],
+                                             d["beta"][:, keep], d["state"])
+    np.testing.assert_array_equal(S, Ss)
+    np.testing.assert_array_equal(y[:, keep], ys)
+    np.testing.assert_array_equal(tape[:, keep], ts)
+    assert np.all(y[:, ~keep] == 0) and np.all(tape[:, ~keep] == 0)
+    assert tape.dtype == np.float32
+
+
+# ------------------------------------------------- acceptance and indexing --
+
+
+def test_match_acceptance_length_doc_example():
+    # DFlashRuntime.swift:130-132
+    assert O.match_acceptance_length([1, 2, 3], [1, 2, 5]) == 2
+    assert O.match_acceptance_length([], []) == 0
+    assert O.match_acceptance_length([7], [7]) == 1
+    assert O.match_acceptance_length([1, 2, 3], [9, 2, 3]) == 0     # later matches do not count
+    assert O.match_acceptance_length([1, 2, 3], [1, 9, 3]) == 1
+
+
+def test_match_acceptance_length_brute_force():
+    rng = np.random.default_rng(0)
+    for _ in range(500):
+        n = int(rng.integers(0, 16))
+        a = rng.integers(0, 3, n)
+        b = rng.integers(0, 3, n)
+        want = 0
+        for x, y in zip(a, b):
+            if x != y:
+                break
+            want += 1
+        assert O.match_acceptance_length(a, b) == want
+
+
+def test_accept_commit_indexing():
+    rng = np.random.default_rng(1)
+    for _ in range(200):
+        V = int(rng.integers(1, 17))
+        staged = int(rng.integers(0, 50))
+        drafted = rng.integers(0, 4, V - 1)
+        posterior = rng.integers(0, 4, V)
+        start = int(rng.integers(0, 1000))
+        r = O.accept_commit(staged, drafted, posterior, start)
+        a = 0
+        while a < V - 1 and drafted[a] == posterior[a]:
+            a += 1
+        assert r["acceptance_len"] == a and 0 <= a <= V - 1
+        assert r["commit_count"] == a + 1
+        assert list(r["committed"]) == [staged] + list(drafted[:a])
+        assert r["staged_next"] == posterior[a]
+        assert r["start"] == start + a + 1
+        assert r["rollback_args"] == {"target_len": start + a + 1, "acceptance_length": a, "drafted_tokens": V - 1}
+
+
+def test_rebuild_conv_state_brute_force():
+    rng = np.random.default_rng(2)
+    B, keep, C, T = 2, 3, 5, 8
+    snap = rng.standard_normal((B, keep, C)).astype(np.float32)
+    qkv = rng.standard_normal((B, T, C)).astype(np.float32)
+    for steps in range(1, T + 1):
+        got = O.rebuild_conv_state(snap, qkv, steps, keep)
+        # the window is the last `keep` inputs seen after `steps` tokens
+        hist = [snap[:, i] for i in range(keep)] + [qkv[:, t] for t in range(steps)]
+        want = np.stack(hist[-keep:], axis=1)
+        np.testing.assert_array_equal(got, want)
+    np.testing.assert_array_equal(O.rebuild_conv_state(None, qkv, 1, keep)[:, :2], 0)
+    # the slice end is clamped (RecurrentRollbackCache.swift:156)
+    assert O.rebuild_conv_state(snap, qkv, T + 2, keep).shape[1] == 1
+
+
+def test_restore_target_cache_actions():
+    caches = [("rollback", 0), ("kv", 116), ("mamba", 0), ("kv", 100)]
+    # partial acceptance: replay nAccepted, trim KV down to targetLen
+    assert O.restore_target_cache_after_acceptance(caches, 104, 3, 15) == [
+        ("rollback", 3), ("trim", 12), ("set_offset", 104), ("none",)]
+    # fully accepted: no replay (DFlashRuntime.swift:194,199-202)
+    assert O.restore_target_cache_after_acceptance(caches, 116, 15, 15)[0] == ("clear",)
+    # draftedTokens == 0 is never "fully accepted"
+    assert O.restore_target_cache_after_acceptance(caches, 101, 0, 0)[0] == ("rollback", 0)
+
+
+def test_rollback_cache_state_machine():
+    d = _gdn(20, B=1, T=8, Hk=2, Hv=4, Dk=8, Dv=8)
+    rng = np.random.default_rng(3)
+    conv0 = rng.standard_normal((1, 3, 10)).astype(np.float32)
+    qkv = rng.standard_normal((1, 8, 10)).astype(np.float32)
+    c = O.RecurrentRollbackCacheOracle()
+    c.slots = [conv0, d["state"]]
+    c.arm_rollback(prefix_len=5)
+    assert c.armed
+    y, S_full, tape = O.gated_delta_ops_with_tape(d["q"], d["k"], d["v"], d["g"], d["beta"], d["state"])
+    c.slots = [qkv[:, -3:], S_full]        # what the verify forward leaves behind
+    c.record_tape(tape, d["k"], d["g"], qkv)
+    c.rollback(n_accepted=2)               # acceptedSteps = 3
+    _, S3, _ = O.gated_delta_ops_with_tape(d["q"][:, :3], d["k"][:, :3], d["v"][:, :3], d["g"][:, :3],
+                                           d["beta"][:, :3], d["state"])
+    np.testing.assert_allclose(c.slots[1], S3, rtol=1e-5, atol=1e-6)
+    np.testing.assert_array_equal(c.slots[0], qkv[:, 0:3])
+    assert not c.armed and c._snapshot is None
+    # rollback without arm is a no-op that clears
+    before = c.slots[1].copy()
+    c.rollback(n_accepted=0)
+    np.testing.assert_array_equal(c.slots[1], before)
+    c.offset = 5
+    assert c.trim(8) == 5 and c.offset == 0
+
+
+# -------------------------------------------------------------------- sdpa --
+
+
+def _sdpa_library(q, k, v, scale):
+    B, Hq, M, D = q.shape
+    Hk, N = k.shape[1:3]
+    kk = np.repeat(k.astype(F64), Hq // Hk, axis=1)
+    vv = np.repeat(v.astype(F64), Hq // Hk, axis=1)
+    s = np.einsum("bhmd,bhnd->bhmn", q.astype(F64), kk) * scale
+    vis = np.arange(N)[None, :] <= (N - M + np.arange(M))[:, None]
+    s = np.where(vis, s, -np.inf)
+    return np.einsum("bhmn,bhnd->bhmd", softmax(s, axis=-1), vv), logsumexp(s, axis=-1)
+
+
+def test_sdpa_matches_library_softmax():
+    q, k, v = O.make_sdpa_inputs(0, B=2, Hq=4, Hk=2, M=16, L=37, D=8)
+    o, lse = O.sdpa_block_causal(q, k, v, 0.3)
+    ow, lw = _sdpa_library(q, k, v, 0.3)
+    np.testing.assert_allclose(o, ow, rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(lse, lw, rtol=1e-12, atol=1e-14)
+
+
+def test_sdpa_invariants():
+    q, k, v = O.make_sdpa_inputs(1, B=1, Hq=4, Hk=2, M=16, L=20, D=8)
+    # constant V -> constant O (rows of the softmax sum to one)
+    o, _ = O.sdpa_block_causal(q, k, np.full_like(v, 2.5), 0.2)
+    np.testing.assert_allclose(o, 2.5, rtol=1e-13)
+    # L = 0: plain causal attention over the block; row 0 sees only key 0
+    q, k, v = O.make_sdpa_inputs(2, B=1, Hq=2, Hk=1, M=16, L=0, D=8)
+    o, lse = O.sdpa_block_causal(q, k, v, 0.5)
+    np.testing.assert_allclose(o[0, :, 0], np.broadcast_to(v[0, 0, 0], (2, 8)), rtol=1e-13)
+    s = np.einsum("hmd,nd->hmn", q[0].astype(F64), k[0, 0].astype(F64)) * 0.5
+    s = np.where(np.tril(np.ones((16, 16), bool)), s, -np.inf)
+    np.testing.assert_allclose(o[0], softmax(s, -1) @ v[0, 0].astype(F64), rtol=1e-12)
+    np.testing.assert_allclose(lse[0], logsumexp(s, -1), rtol=1e-12)
+    # GQA: query heads 0,1 read kv head 0 and heads 2,3 read kv head 1
+    q, k, v = O.make_sdpa_inputs(3, B=1, Hq=4, Hk=2, M=16, L=8, D=8)
+    v2 = v.copy()
+    v2[:, 1] += 1.0
+    o1, _ = O.sdpa_block_causal(q, k, v, 0.3)
+    o2, _ = O.sdpa_block_causal(q, k, v2, 0.3)
+    np.testing.assert_allclose(o2[:, :2], o1[:, :2], rtol=1e-13)
+    np.testing.assert_allclose(o2[:, 2:], o1[:, 2:] + 1.0, rtol=1e-12)
+
+
+def test_sdpa_additive_mask():
+    q, k, v = O.make_sdpa_inputs(4, B=1, Hq=2, Hk=1, M=16, L=16, D=8)
+    mask = np.zeros((1, 2, 16, 32))
+    mask[..., :5] = -np.inf                               # hide the first five keys
+    o, _ = O.sdpa_block_causal(q, k, v, 0.3, mask)
+    ow, _ = O.sdpa_block_causal(q, k[:, :, 5:], v[:, :, 5:], 0.3)
+    np.testing.assert_allclose(o, ow, rtol=1e-12)
+
+
+@pytest.mark.parametrize("blocks", [32, 64])
+def test_sdpa_2pass_agrees_with_single_pass(blocks):
+    q, k, v = O.make_sdpa_inputs(5, B=1, Hq=4, Hk=2, M=16, L=200, D=16)
+    want, _ = O.sdpa_block_causal(q, k, v, 0.25)
+    exact = O.sdpa_2pass(q, k, v, 0.25, blocks, partial_dtype="f32")
+    np.testing.assert_allclose(exact, want, rtol=2e-5, atol=2e-6)
+    rounded = O.sdpa_2pass(q, k, v, 0.25, blocks, partial_dtype="bf16")
+    np.testing.assert_allclose(rounded, want, rtol=2e-2, atol=2e-2)
+
+
+# ---------------------------------------------------------------- C oracle --
+
+
+@pytest.mark.parametrize("variant", ["fused", "opbyop"])
+@pytest.mark.parametrize("vec", [False, True])
+@pytest.mark.parametrize("masked", [False, True])
+def test_c_oracle_matches_numpy_oracle(variant, vec, masked):
+    from oracle import c_oracle
+
+    d = _gdn(30, B=2, T=5, Hk=2, Hv=4, Dk=16, Dv=8, vec=vec)
+    mask = np.array([[1, 0, 1, 1, 0], [0, 1, 1, 0, 1]], np.float32) if masked else None
+    got = c_oracle.tape_replay(d["tape"], d["k"], d["g"], d["state"], mask, variant=variant)
+    want = O.tape_replay_ops(d["tape"], d["k"], d["g"], d["state"], mask, dtype=F64)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+    y, S, tape = c_oracle.gated_delta(d["q"], d["k"], d["v"], d["g"], d["beta"], d["state"], mask,
+                                      variant=variant)
+    yw, Sw, tw = O.gated_delta_ops_with_tape(d["q"], d["k"], d["v"], d["g"], d["beta"], d["state"], mask,
+                                             dtype=F64)
+    np.testing.assert_allclose(y, yw, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(S, Sw, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(tape, tw, rtol=1e-4, atol=1e-5)
+
+
+def test_c_oracle_sdpa_and_accept():
+    from oracle import c_oracle
+
+    q, k, v = O.make_sdpa_inputs(6, B=2, Hq=4, Hk=2, M=16, L=50, D=16)
+    o, lse = c_oracle.sdpa_block_causal(q, k, v, 0.25)
+    ow, lw = O.sdpa_block_causal(q, k, v, 0.25)
+    np.testing.assert_allclose(o, ow, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(lse, lw, rtol=1e-5, atol=1e-5)
+    assert c_oracle.match_acceptance_length([1, 2, 3], [1, 2, 5]) == 2
+    assert c_oracle.match_acceptance_length([], []) == 0
