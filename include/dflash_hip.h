@@ -1,0 +1,199 @@
+/*
+ * dflash_hip.h — C ABI of the MI355X (gfx950) DFlash speculative-verify kernels.
+ *
+ * One shared library, libdflash_hip.so.  Plain pointers and sizes only; no C++
+ * types, no exceptions and no aborts cross this boundary.  Every array argument
+ * is DEVICE memory owned by the caller unless a comment says "host".  Inputs are
+ * never written, outputs are never allocated or freed here, and state_in may not
+ * alias state_out.  All work is enqueued on the caller's stream (`stream` is a
+ * hipStream_t passed as void*; NULL is the default stream) and the calls return
+ * without synchronising.  The library is re-entrant.
+ *
+ * Return value of every `int` function:
+ *    0                  work enqueued (DFLASH_OK)
+ *    DFLASH_UNSUPPORTED the shape/dtype is outside what the kernels cover; nothing
+ *                       was launched.  This is the analogue of the reference
+ *                       returning nil / taking its ops path
+ *                       (Sources/DFlash/DFlashKernels.swift:271-273, :744-758).
+ *    DFLASH_INVALID     inconsistent arguments (NULL pointer, non-positive size,
+ *                       Hv not a multiple of Hk, workspace too small ...).
+ *    < 0                minus the hipError_t of a failed HIP call.
+ * dflash_last_error() returns a thread-local description of the last failure.
+ *
+ * Layouts (row-major, last index fastest), as in the reference:
+ *    q, k          [B, T, Hk, Dk]
+ *    v, y, tape    [B, T, Hv, Dv]
+ *    g             [B, T, Hv]        (g_ndim == 3, one decay per head)
+ *                  [B, T, Hv, Dk]    (g_ndim == 4, one decay per key channel)
+ *    beta          [B, T, Hv]
+ *    state         [B, Hv, Dv, Dk]
+ *    mask          [B, T]            a step runs when mask > 0.5
+ *    g is the MULTIPLICATIVE decay (state * g), not its logarithm.
+ *    Value head hv reads key head hv / (Hv / Hk).
+ */
+#ifndef DFLASH_HIP_H
+#define DFLASH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DFLASH_OK 0
+#define DFLASH_UNSUPPORTED 1
+#define DFLASH_INVALID 2
+
+/* Element types. */
+#define DFLASH_F32 0
+#define DFLASH_BF16 1
+#define DFLASH_F16 2
+#define DFLASH_U8 3 /* masks only */
+
+#define DFLASH_MAX_BATCHED_LAYERS 64
+
+int dflash_version(void);
+const char* dflash_last_error(void);
+
+/* Loads the code object on the current device and sizes the kernels' LDS
+ * budgets.  Optional: every entry point does this on first use.  Thread-safe. */
+int dflash_init(void);
+
+/* ------------------------------------------------------------------------
+ * Tape replay.  Replaces DFlashKernels.tapeReplayKernel
+ * (Sources/DFlash/DFlashKernels.swift:252-301; Metal source :43-81; ops
+ * restatement :371-407).  For t < T:  S <- S * g_t + tape_t (x) k_t ; a masked
+ * step leaves S untouched.  The caller passes the accepted prefix
+ * (T = nAccepted + 1, RecurrentRollbackCache.swift:115-125).
+ *   tape_dtype : DFLASH_F32 (the recorded innovation tape) or == in_dtype
+ *   in_dtype   : type of k and g
+ *   state_dtype: DFLASH_F32, or == in_dtype in which case S is re-rounded to
+ *                that type after every step as the Metal kernel does (:70).
+ *   mask       : NULL, or [B,T] of mask_dtype (F32/BF16/F16/U8)
+ * T == 0 copies state_in to state_out.
+ * ---------------------------------------------------------------------- */
+int dflash_tape_replay(void* stream,
+                       const void* tape, int tape_dtype,
+                       const void* k, const void* g, int in_dtype, int g_ndim,
+                       const void* state_in, void* state_out, int state_dtype,
+                       const void* mask, int mask_dtype,
+                       int B, int T, int Hk, int Hv, int Dk, int Dv);
+
+/* Replays `n_layers` independent caches in ONE launch.  Replaces the serial
+ * loop over caches in DFlashRuntime.restoreTargetCacheAfterAcceptance
+ * (Sources/DFlash/DFlashRuntime.swift:197-205), where every
+ * RecurrentRollbackCache.rollback issues its own kernel.
+ * The pointer arrays are HOST arrays of n_layers device pointers (copied into
+ * the launch); all layers share shapes, dtypes and T_tape (the recorded tape
+ * length, i.e. the stride-defining T of tape/k/g).
+ * Steps replayed: `steps` when steps_dev == NULL, else min(*steps_dev, T_tape)
+ * read on the device (an int32), which lets the accept kernel feed the replay
+ * without a host round trip.  When skip_if_full != 0 and the step count equals
+ * T_tape the kernel writes nothing: a fully accepted block keeps the state
+ * the verify forward left in state_out (DFlashRuntime.swift:194,199-202).
+ * n_layers <= DFLASH_MAX_BATCHED_LAYERS. */
+int dflash_tape_replay_batched(void* stream, int n_layers,
+                               const void* const* tape, int tape_dtype,
+                               const void* const* k, const void* const* g, int in_dtype, int g_ndim,
+                               const void* const* state_in, void* const* state_out, int state_dtype,
+                               int steps, const int32_t* steps_dev, int skip_if_full,
+                               int B, int T_tape, int Hk, int Hv, int Dk, int Dv);
+
+/* ------------------------------------------------------------------------
+ * GatedDelta forward that records the innovation tape.  Replaces
+ * DFlashKernels.gatedDeltaKernelWithTape and the DFlashKernelProvider method of
+ * the same name (DFlashKernels.swift:316-367, Metal :122-199, ops :409-466;
+ * Sources/DFlash/DFlashKernelProvider.swift:8-14).  Per step:
+ *   S' = S * g ; m = S' k ; delta = (v - m) * beta ; S = S' + delta (x) k ;
+ *   y = S q.   A masked step keeps S and writes y = 0, delta = 0.
+ *   q,k,v,g,beta : in_dtype          y : in_dtype        tape_out : float32
+ *   state        : state_dtype (F32, or == in_dtype with per-step re-rounding,
+ *                  DFlashKernels.swift:183-186)
+ * ---------------------------------------------------------------------- */
+int dflash_gated_delta_tape(void* stream,
+                            const void* q, const void* k, const void* v,
+                            const void* g, int g_ndim, const void* beta, int in_dtype,
+                            const void* state_in, void* state_out, int state_dtype,
+                            void* y, float* tape_out,
+                            const void* mask, int mask_dtype,
+                            int B, int T, int Hk, int Hv, int Dk, int Dv);
+
+/* ------------------------------------------------------------------------
+ * Block-causal batched GQA SDPA for the verify block.  Replaces
+ * DFlashKernels.batchedSDPA2Pass (DFlashKernels.swift:737-815; Metal partials
+ * :563-649, reduce :661-720); unlike it, covers every shape sdpaFallback
+ * (:818-828) would be asked for at M == 16, so DFLASH_UNSUPPORTED mirrors the
+ * reference's nil.
+ *   q    [B, Hq, M, D]   contiguous, M must be 16 (:755)
+ *   k,v  element (b, hk, n, d) at  b*kv_batch_stride + hk*kv_head_stride + n*D + d
+ *        (strides in elements; a dense [B,Hk,N,D] has head stride N*D, batch
+ *        stride Hk*N*D; a preallocated cache passes its capacity instead)
+ *   N    number of keys INCLUDING the M block tokens; query row i sees keys
+ *        0 .. N-M+i (:614).  hk = hq / (Hq/Hk) (:575).
+ *   kv_len_dev  NULL, or device int32[B]: per-sequence key counts (ragged
+ *        batches, or a count produced on the device); each must be in [M, N].
+ *   out  [B, Hq, M, D] of `dtype`;  lse  NULL or float32 [B, Hq, M] receiving
+ *        max + log(sum exp) of the scaled, masked scores (natural log).
+ *   dtype DFLASH_BF16 or DFLASH_F16 (:756); D in {128, 256} (:757).
+ *   workspace  device scratch of at least dflash_sdpa_workspace_bytes(...)
+ *        bytes, 256-byte aligned; contents are undefined afterwards.
+ * ---------------------------------------------------------------------- */
+size_t dflash_sdpa_workspace_bytes(int B, int Hq, int Hk, int M, int N, int D);
+
+int dflash_sdpa_block_causal(void* stream,
+                             const void* q, const void* k, const void* v,
+                             void* out, float* lse, int dtype, float scale,
+                             int B, int Hq, int Hk, int M, int N, int D,
+                             int64_t kv_batch_stride, int64_t kv_head_stride,
+                             const int32_t* kv_len_dev,
+                             void* workspace, size_t workspace_bytes);
+
+/* ------------------------------------------------------------------------
+ * Acceptance.  dflash_match_acceptance_length replaces
+ * DFlashRuntime.matchAcceptanceLength (Sources/DFlash/DFlashRuntime.swift:
+ * 133-142): out[0] = number of leading positions with drafted[i] == posterior[i]
+ * (0 when n == 0).  Tokens are uint32 on the device; out is a device int32.
+ *
+ * dflash_accept_commit does one verify cycle's integer bookkeeping on the
+ * device (DFlashRuntime.swift:490-493, :525-530, :544-547, :571):
+ *   verify_ids [V] = [staged_first, drafted...] ; posterior [V]
+ *   out[0] = acceptanceLen = leading matches of verify_ids[1:] vs posterior[:V-1]
+ *   out[1] = commitCount   = 1 + acceptanceLen  (= steps to replay)
+ *   out[2] = stagedFirstNext = posterior[acceptanceLen]
+ *   out[3] = *start_inout += commitCount (start_inout may be NULL -> commitCount)
+ * ---------------------------------------------------------------------- */
+int dflash_match_acceptance_length(void* stream, const uint32_t* drafted, const uint32_t* posterior,
+                                   int n, int32_t* out);
+int dflash_accept_commit(void* stream, const uint32_t* verify_ids, const uint32_t* posterior, int V,
+                         int32_t* start_inout, int32_t* out4);
+
+/* ------------------------------------------------------------------------
+ * Conv-state rebuild after rollback.  Replaces
+ * RecurrentRollbackCache.rebuildConvState (Sources/DFlash/
+ * RecurrentRollbackCache.swift:139-158):
+ *   out[b, j, :] = concat(snapshot_conv [B,keep,C], tape_qkv [B,T,C])[b, s + j, :]
+ * for j < min(keep, keep + T - s), s = accepted_steps (or *steps_dev when not
+ * NULL).  snapshot_conv == NULL stands for zeros (:147-152).  elem_bytes is the
+ * element size (2 or 4).  Rows past the clamp are left untouched; the number of
+ * valid rows is min(keep, keep + T - s) as in the reference's clamped slice.
+ * ---------------------------------------------------------------------- */
+int dflash_rebuild_conv_state(void* stream, const void* snapshot_conv, const void* tape_qkv, void* out,
+                              int B, int keep, int T, int C, int elem_bytes,
+                              int accepted_steps, const int32_t* steps_dev);
+
+/* ------------------------------------------------------------------------
+ * KV append for an attention layer at verify (the KVCacheSimple.update the
+ * reference delegates to mlx-swift-lm, trimmed by DFlashRuntime.swift:212-218):
+ * copies k_new/v_new [B, Hk, M, D] to rows [offset, offset+M) of a cache laid out
+ * like k/v above.  offset comes from *offset_dev when not NULL.
+ * ---------------------------------------------------------------------- */
+int dflash_kv_append(void* stream, void* k_cache, void* v_cache, const void* k_new, const void* v_new,
+                     int B, int Hk, int M, int D, int elem_bytes,
+                     int64_t kv_batch_stride, int64_t kv_head_stride,
+                     int offset, const int32_t* offset_dev, int capacity);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DFLASH_HIP_H */

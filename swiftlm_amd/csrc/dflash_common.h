@@ -1,0 +1,136 @@
+// Shared helpers for the gfx950 DFlash kernels: element types, error plumbing,
+// wave-level reductions.  Internal to the library.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/dflash_hip.h"
+
+namespace dflash {
+
+// ---- error plumbing ------------------------------------------------------
+
+void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+
+#define DFLASH_HIP_TRY(expr)                                                        \
+    do {                                                                            \
+        hipError_t _e = (expr);                                                     \
+        if (_e != hipSuccess) {                                                     \
+            ::dflash::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), \
+                                __FILE__, __LINE__);                                \
+            return -(int)_e;                                                        \
+        }                                                                           \
+    } while (0)
+
+#define DFLASH_REQUIRE(cond, ...)              \
+    do {                                       \
+        if (!(cond)) {                         \
+            ::dflash::set_error(__VA_ARGS__);  \
+            return DFLASH_INVALID;             \
+        }                                      \
+    } while (0)
+
+#define DFLASH_SUPPORTED(cond, ...)            \
+    do {                                       \
+        if (!(cond)) {                         \
+            ::dflash::set_error(__VA_ARGS__);  \
+            return DFLASH_UNSUPPORTED;         \
+        }                                      \
+    } while (0)
+
+int ensure_init();           // per-device one-time setup; 0 or negative hip error
+int num_compute_units();     // of the current device (cached)
+
+inline int dtype_size(int dt) {
+    switch (dt) {
+        case DFLASH_F32: return 4;
+        case DFLASH_BF16: return 2;
+        case DFLASH_F16: return 2;
+        case DFLASH_U8: return 1;
+        default: return 0;
+    }
+}
+
+// ---- element types -------------------------------------------------------
+
+struct bf16_t { uint16_t bits; };
+struct f16_t { _Float16 v; };
+
+__device__ __forceinline__ float to_float(float x) { return x; }
+__device__ __forceinline__ float to_float(bf16_t x) { return __uint_as_float(((uint32_t)x.bits) << 16); }
+__device__ __forceinline__ float to_float(f16_t x) { return (float)x.v; }
+
+// round-to-nearest-even, NaN preserved
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ T from_float(float f);
+template <> __device__ __forceinline__ float from_float<float>(float f) { return f; }
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float f) { return bf16_t{f32_to_bf16_bits(f)}; }
+template <> __device__ __forceinline__ f16_t from_float<f16_t>(float f) { return f16_t{(_Float16)f}; }
+
+// value after a round trip through T (identity for float)
+template <typename T> __device__ __forceinline__ float requant(float f) { return to_float(from_float<T>(f)); }
+template <> __device__ __forceinline__ float requant<float>(float f) { return f; }
+
+// 4 consecutive elements -> float4 (pointer aligned to 4 elements)
+__device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4(const bf16_t* p) {
+    uint2 u = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
+                       __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
+}
+__device__ __forceinline__ float4 load4(const f16_t* p) {
+    return make_float4((float)p[0].v, (float)p[1].v, (float)p[2].v, (float)p[3].v);
+}
+__device__ __forceinline__ void store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16_t* p, float4 v) {
+    uint2 u;
+    u.x = (uint32_t)f32_to_bf16_bits(v.x) | ((uint32_t)f32_to_bf16_bits(v.y) << 16);
+    u.y = (uint32_t)f32_to_bf16_bits(v.z) | ((uint32_t)f32_to_bf16_bits(v.w) << 16);
+    *reinterpret_cast<uint2*>(p) = u;
+}
+__device__ __forceinline__ void store4(f16_t* p, float4 v) {
+    p[0].v = (_Float16)v.x; p[1].v = (_Float16)v.y; p[2].v = (_Float16)v.z; p[3].v = (_Float16)v.w;
+}
+
+// mask element of run-time type -> "this step runs"
+__device__ __forceinline__ bool mask_on(const void* mask, int mask_dtype, int idx) {
+    float m;
+    switch (mask_dtype) {
+        case DFLASH_F32: m = reinterpret_cast<const float*>(mask)[idx]; break;
+        case DFLASH_BF16: m = to_float(reinterpret_cast<const bf16_t*>(mask)[idx]); break;
+        case DFLASH_F16: m = to_float(reinterpret_cast<const f16_t*>(mask)[idx]); break;
+        default: m = (float)reinterpret_cast<const uint8_t*>(mask)[idx]; break;
+    }
+    return m > 0.5f;
+}
+
+// ---- cross-lane sums inside one 16-lane DPP row ---------------------------
+// Data-parallel-primitive controls of GFX9: quad_perm, row_half_mirror, row_mirror.
+
+template <int CTRL> __device__ __forceinline__ float dpp_add(float x) {
+    int y = __builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false);
+    return x + __int_as_float(y);
+}
+
+// Sum over groups of LANES (4, 8 or 16) consecutive lanes; every lane of the
+// group receives the total.
+template <int LANES> __device__ __forceinline__ float group_sum(float x) {
+    static_assert(LANES == 4 || LANES == 8 || LANES == 16, "group must fit one DPP row");
+    x = dpp_add<0xB1>(x);                          // quad_perm [1,0,3,2]
+    x = dpp_add<0x4E>(x);                          // quad_perm [2,3,0,1]
+    if (LANES >= 8) x = dpp_add<0x141>(x);         // row_half_mirror
+    if (LANES >= 16) x = dpp_add<0x140>(x);        // row_mirror
+    return x;
+}
+
+}  // namespace dflash

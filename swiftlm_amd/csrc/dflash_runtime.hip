@@ -1,0 +1,194 @@
+// Library plumbing (init, error text) and the small integer/byte kernels of the
+// verify step: acceptance length, accept/commit bookkeeping, conv-state
+// rebuild, KV append.
+
+#include <stdarg.h>
+#include <string.h>
+
+#include <mutex>
+
+#include "dflash_common.h"
+
+namespace dflash {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+static std::mutex g_init_mu;
+static int g_cus[64];
+static bool g_ready[64];
+
+int ensure_init() {
+    int dev = 0;
+    DFLASH_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) { set_error("device index %d out of range", dev); return DFLASH_INVALID; }
+    std::lock_guard<std::mutex> lock(g_init_mu);
+    if (g_ready[dev]) return 0;
+    hipDeviceProp_t prop;
+    DFLASH_HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        set_error("this library is built for gfx950 only; device %d is %s", dev, prop.gcnArchName);
+        return DFLASH_UNSUPPORTED;
+    }
+    g_cus[dev] = prop.multiProcessorCount;
+    g_ready[dev] = true;
+    return 0;
+}
+
+int num_compute_units() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64 || !g_ready[dev]) return 256;
+    return g_cus[dev];
+}
+
+// ---- acceptance ------------------------------------------------------------
+
+// One wave.  Leading-match count = index of the first mismatch (n if none);
+// equals sum(cumprod(drafted == posterior)) (DFlashRuntime.swift:139-141).
+__device__ __forceinline__ int leading_matches(const uint32_t* a, const uint32_t* b, int n) {
+    const int lane = threadIdx.x;
+    int first = n;
+    for (int base = 0; base < n; base += 64) {
+        const int i = base + lane;
+        const bool mismatch = i < n && a[i] != b[i];
+        const unsigned long long bal = __builtin_amdgcn_ballot_w64(mismatch);
+        if (bal) { first = base + __builtin_ctzll(bal); break; }   // uniform
+    }
+    return first;
+}
+
+__global__ __launch_bounds__(64) void match_acceptance_kernel(const uint32_t* drafted, const uint32_t* posterior,
+                                                              int n, int32_t* out) {
+    const int acc = leading_matches(drafted, posterior, n);
+    if (threadIdx.x == 0) out[0] = acc;
+}
+
+__global__ __launch_bounds__(64) void accept_commit_kernel(const uint32_t* verify_ids, const uint32_t* posterior, int V,
+                                                           int32_t* start_inout, int32_t* out4) {
+    // drafted = verify_ids[1:], posterior[:V-1]  (DFlashRuntime.swift:525-530)
+    const int acc = V > 1 ? leading_matches(verify_ids + 1, posterior, V - 1) : 0;
+    if (threadIdx.x == 0) {
+        const int commit = 1 + acc;                       // :544
+        out4[0] = acc;
+        out4[1] = commit;
+        out4[2] = (int32_t)posterior[acc];                // :547
+        int start = commit;
+        if (start_inout) { start += *start_inout; *start_inout = start; }   // :571
+        out4[3] = start;
+    }
+}
+
+// ---- conv-state rebuild ----------------------------------------------------
+
+// out[b, j, :] = concat(snapshot [B,keep,C], qkv [B,T,C])[b, s + j, :], 16-byte pieces.
+__global__ __launch_bounds__(256) void rebuild_conv_kernel(const uint4* snap, const uint4* qkv, uint4* out, int keep,
+                                                           int T, int C16, int steps, const int32_t* steps_dev) {
+    int s = steps_dev ? *steps_dev : steps;
+    s = s < 0 ? 0 : s;
+    const int b = blockIdx.z, j = blockIdx.y;
+    const int src = s + j;
+    if (src >= keep + T) return;     // clamped slice end (RecurrentRollbackCache.swift:156)
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < C16; i += gridDim.x * blockDim.x) {
+        uint4 val;
+        if (src < keep) val = snap ? snap[((size_t)b * keep + src) * C16 + i] : make_uint4(0, 0, 0, 0);
+        else val = qkv[((size_t)b * T + (src - keep)) * C16 + i];
+        out[((size_t)b * keep + j) * C16 + i] = val;
+    }
+}
+
+// ---- KV append -------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void kv_append_kernel(uint4* k_cache, uint4* v_cache, const uint4* k_new,
+                                                        const uint4* v_new, int Hk, int M, int D16, long batch_stride16,
+                                                        long head_stride16, int offset, const int32_t* offset_dev,
+                                                        int capacity) {
+    int off = offset_dev ? *offset_dev : offset;
+    if (off < 0 || off + M > capacity) return;   // never write outside the cache
+    const int bh = blockIdx.y;
+    const int b = bh / Hk, hk = bh % Hk;
+    const int per = M * D16;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < per; i += gridDim.x * blockDim.x) {
+        const size_t dst = (size_t)b * batch_stride16 + (size_t)hk * head_stride16 + (size_t)off * D16 + i;
+        const size_t src = (size_t)bh * per + i;
+        k_cache[dst] = k_new[src];
+        v_cache[dst] = v_new[src];
+    }
+}
+
+}  // namespace dflash
+
+using namespace dflash;
+
+extern "C" int dflash_version(void) { return 100; }
+extern "C" const char* dflash_last_error(void) { return g_err; }
+extern "C" int dflash_init(void) { return ensure_init(); }
+
+extern "C" int dflash_match_acceptance_length(void* stream, const uint32_t* drafted, const uint32_t* posterior, int n,
+                                              int32_t* out) {
+    int rc = ensure_init();
+    if (rc) return rc;
+    DFLASH_REQUIRE(out && n >= 0 && (n == 0 || (drafted && posterior)), "match_acceptance_length: bad arguments");
+    hipLaunchKernelGGL(match_acceptance_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, drafted, posterior, n, out);
+    DFLASH_HIP_TRY(hipGetLastError());
+    return DFLASH_OK;
+}
+
+extern "C" int dflash_accept_commit(void* stream, const uint32_t* verify_ids, const uint32_t* posterior, int V,
+                                    int32_t* start_inout, int32_t* out4) {
+    int rc = ensure_init();
+    if (rc) return rc;
+    DFLASH_REQUIRE(verify_ids && posterior && out4 && V >= 1, "accept_commit: bad arguments");
+    hipLaunchKernelGGL(accept_commit_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, verify_ids, posterior, V,
+                       start_inout, out4);
+    DFLASH_HIP_TRY(hipGetLastError());
+    return DFLASH_OK;
+}
+
+extern "C" int dflash_rebuild_conv_state(void* stream, const void* snapshot_conv, const void* tape_qkv, void* out, int B,
+                                         int keep, int T, int C, int elem_bytes, int accepted_steps,
+                                         const int32_t* steps_dev) {
+    int rc = ensure_init();
+    if (rc) return rc;
+    DFLASH_REQUIRE(tape_qkv && out && B > 0 && keep > 0 && T >= 0 && C > 0, "rebuild_conv_state: bad arguments");
+    DFLASH_REQUIRE(elem_bytes == 2 || elem_bytes == 4, "rebuild_conv_state: element size must be 2 or 4");
+    DFLASH_REQUIRE(accepted_steps >= 0, "rebuild_conv_state: negative accepted_steps");
+    DFLASH_REQUIRE(((long)C * elem_bytes) % 16 == 0, "rebuild_conv_state: row of %d x %d bytes is not a multiple of 16", C, elem_bytes);
+    DFLASH_REQUIRE(((uintptr_t)snapshot_conv | (uintptr_t)tape_qkv | (uintptr_t)out) % 16 == 0, "rebuild_conv_state: pointers must be 16-byte aligned");
+    DFLASH_REQUIRE(keep <= 65535 && B <= 65535, "rebuild_conv_state: keep or B too large");
+    const int C16 = (int)(((long)C * elem_bytes) / 16);
+    dim3 grid((C16 + 255) / 256, keep, B);
+    hipLaunchKernelGGL(rebuild_conv_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const uint4*)snapshot_conv,
+                       (const uint4*)tape_qkv, (uint4*)out, keep, T, C16, accepted_steps, steps_dev);
+    DFLASH_HIP_TRY(hipGetLastError());
+    return DFLASH_OK;
+}
+
+extern "C" int dflash_kv_append(void* stream, void* k_cache, void* v_cache, const void* k_new, const void* v_new, int B,
+                                int Hk, int M, int D, int elem_bytes, int64_t kv_batch_stride, int64_t kv_head_stride,
+                                int offset, const int32_t* offset_dev, int capacity) {
+    int rc = ensure_init();
+    if (rc) return rc;
+    DFLASH_REQUIRE(k_cache && v_cache && k_new && v_new, "kv_append: null pointer");
+    DFLASH_REQUIRE(B > 0 && Hk > 0 && M > 0 && D > 0 && capacity > 0, "kv_append: non-positive dimension");
+    DFLASH_REQUIRE(elem_bytes == 2 || elem_bytes == 4, "kv_append: element size must be 2 or 4");
+    DFLASH_REQUIRE(((long)D * elem_bytes) % 16 == 0, "kv_append: row bytes must be a multiple of 16");
+    DFLASH_REQUIRE((kv_batch_stride * elem_bytes) % 16 == 0 && (kv_head_stride * elem_bytes) % 16 == 0, "kv_append: strides must be 16-byte multiples");
+    DFLASH_REQUIRE(kv_head_stride >= (int64_t)capacity * D, "kv_append: head stride smaller than capacity*D");
+    DFLASH_REQUIRE(kv_batch_stride >= (int64_t)(Hk - 1) * kv_head_stride + (int64_t)capacity * D, "kv_append: batch stride too small");
+    DFLASH_REQUIRE(offset_dev || (offset >= 0 && offset + M <= capacity), "kv_append: rows [%d, %d) outside capacity %d", offset, offset + M, capacity);
+    DFLASH_REQUIRE(((uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)k_new | (uintptr_t)v_new) % 16 == 0, "kv_append: pointers must be 16-byte aligned");
+    DFLASH_REQUIRE((long)B * Hk <= 65535, "kv_append: B*Hk too large");
+    const int D16 = (int)(((long)D * elem_bytes) / 16);
+    dim3 grid((M * D16 + 255) / 256, B * Hk);
+    hipLaunchKernelGGL(kv_append_kernel, grid, dim3(256), 0, (hipStream_t)stream, (uint4*)k_cache, (uint4*)v_cache,
+                       (const uint4*)k_new, (const uint4*)v_new, Hk, M, D16, (long)(kv_batch_stride * elem_bytes / 16),
+                       (long)(kv_head_stride * elem_bytes / 16), offset, offset_dev, capacity);
+    DFLASH_HIP_TRY(hipGetLastError());
+    return DFLASH_OK;
+}

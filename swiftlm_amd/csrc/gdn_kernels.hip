@@ -1,0 +1,446 @@
+// GatedDelta recurrent-state kernels for gfx950: tape replay and the forward
+// pass that records the innovation tape.
+//
+// Both recurrences are independent per state row (b, hv, dv): a row of Dk
+// floats is updated by rank-1 terms that only need k_t (shared by the head),
+// the row's own delta_t and the head's decay.  The kernels therefore tile a
+// head over Dv across workgroups (one head alone would occupy 32 of 256 CUs),
+// keep each row slice in VGPRs for all T steps, and stage the per-step
+// operands (k, q, v/tape slice, g, beta, mask) through LDS once per chunk of
+// steps so the serial t-loop never waits on global memory.
+//
+// Semantics follow Sources/DFlash/DFlashKernels.swift: Metal kernels :43-81 and
+// :122-199, ops restatements :371-407 and :409-466.
+
+#include "dflash_common.h"
+
+namespace dflash {
+
+constexpr int kThreads = 256;
+
+// 4 consecutive elements of run-time type -> float4
+__device__ __forceinline__ float4 load4_rt(const void* base, int dtype, size_t idx) {
+    switch (dtype) {
+        case DFLASH_F32: return load4(reinterpret_cast<const float*>(base) + idx);
+        case DFLASH_BF16: return load4(reinterpret_cast<const bf16_t*>(base) + idx);
+        default: return load4(reinterpret_cast<const f16_t*>(base) + idx);
+    }
+}
+__device__ __forceinline__ float load1_rt(const void* base, int dtype, size_t idx) {
+    switch (dtype) {
+        case DFLASH_F32: return reinterpret_cast<const float*>(base)[idx];
+        case DFLASH_BF16: return to_float(reinterpret_cast<const bf16_t*>(base)[idx]);
+        default: return to_float(reinterpret_cast<const f16_t*>(base)[idx]);
+    }
+}
+__device__ __forceinline__ void store1_rt(void* base, int dtype, size_t idx, float v) {
+    switch (dtype) {
+        case DFLASH_F32: reinterpret_cast<float*>(base)[idx] = v; break;
+        case DFLASH_BF16: reinterpret_cast<bf16_t*>(base)[idx] = from_float<bf16_t>(v); break;
+        default: reinterpret_cast<f16_t*>(base)[idx] = from_float<f16_t>(v); break;
+    }
+}
+
+// ===========================================================================
+// Tape replay
+// ===========================================================================
+
+struct ReplayBatch {
+    const void* tape[DFLASH_MAX_BATCHED_LAYERS];
+    const void* k[DFLASH_MAX_BATCHED_LAYERS];
+    const void* g[DFLASH_MAX_BATCHED_LAYERS];
+    const void* state_in[DFLASH_MAX_BATCHED_LAYERS];
+    void* state_out[DFLASH_MAX_BATCHED_LAYERS];
+};
+
+struct ReplayArgs {
+    const void* mask;        // [B,T_tape] or null
+    const int32_t* steps_dev;
+    int mask_dtype, tape_dtype, in_dtype;
+    int steps, skip_if_full;
+    int T_tape, Hk, Hv, Dv;
+};
+
+constexpr int kReplayChunk = 32;  // steps staged in LDS at a time (16 for Dk = 256)
+
+// One thread owns 4 consecutive key channels of NR state rows.  DK/4 threads
+// span a row, so a 256-thread workgroup covers RPP = 1024/DK rows per pass and
+// NR passes.  Grid: x = Dv tiles, y = b*Hv + hv, z = layer.
+template <typename StateT, bool VEC_G, int DK, int NR>
+__global__ __launch_bounds__(kThreads) void tape_replay_kernel(ReplayBatch P, ReplayArgs A) {
+    constexpr int TPR = DK / 4;
+    constexpr int RPP = kThreads / TPR;
+    constexpr int ROWS = RPP * NR;
+    constexpr int TC = DK >= 256 ? kReplayChunk / 2 : kReplayChunk;   // keeps static LDS under 64 KB
+
+    __shared__ float k_s[TC][DK];
+    __shared__ float g_s[VEC_G ? TC : 1][VEC_G ? DK : TC];
+    __shared__ float d_s[TC][ROWS];
+    __shared__ int on_s[TC];
+
+    const int layer = blockIdx.z;
+    const int bh = blockIdx.y;
+    const int b = bh / A.Hv, hv = bh % A.Hv;
+    const int hk = hv / (A.Hv / A.Hk);
+    const int row0 = blockIdx.x * ROWS;
+    const int tid = threadIdx.x;
+    const int c4 = (tid % TPR) * 4;
+    const int rsub = tid / TPR;
+
+    int n = A.steps_dev ? *A.steps_dev : A.steps;
+    n = n < 0 ? 0 : (n > A.T_tape ? A.T_tape : n);
+    if (A.skip_if_full && n == A.T_tape) return;   // uniform over the grid
+
+    const StateT* s_in = reinterpret_cast<const StateT*>(P.state_in[layer]) + (size_t)bh * A.Dv * DK;
+    StateT* s_out = reinterpret_cast<StateT*>(P.state_out[layer]) + (size_t)bh * A.Dv * DK;
+    const void* tape = P.tape[layer];
+    const void* kk = P.k[layer];
+    const void* gg = P.g[layer];
+
+    float4 s[NR];
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+        const int r = row0 + rsub + RPP * i;
+        s[i] = r < A.Dv ? load4(s_in + (size_t)r * DK + c4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+
+    for (int t0 = 0; t0 < n; t0 += TC) {
+        const int tc = (n - t0) < TC ? (n - t0) : TC;
+        if (t0) __syncthreads();
+        // ---- stage this chunk's operands as float ----
+        for (int i = tid; i < tc * TPR; i += kThreads) {
+            const int t = i / TPR, c = (i % TPR) * 4;
+            const size_t bt = (size_t)b * A.T_tape + t0 + t;
+            store4(&k_s[t][c], load4_rt(kk, A.in_dtype, (bt * A.Hk + hk) * DK + c));
+            if (VEC_G) store4(&g_s[t][c], load4_rt(gg, A.in_dtype, (bt * A.Hv + hv) * DK + c));
+        }
+        for (int i = tid; i < tc * ROWS; i += kThreads) {
+            const int t = i / ROWS, r = i % ROWS;
+            const size_t bt = (size_t)b * A.T_tape + t0 + t;
+            d_s[t][r] = (row0 + r) < A.Dv ? load1_rt(tape, A.tape_dtype, (bt * A.Hv + hv) * A.Dv + row0 + r) : 0.f;
+        }
+        if (tid < tc) {
+            const size_t bt = (size_t)b * A.T_tape + t0 + tid;
+            if (!VEC_G) g_s[0][tid] = load1_rt(gg, A.in_dtype, bt * A.Hv + hv);
+            on_s[tid] = A.mask ? (int)mask_on(A.mask, A.mask_dtype, (int)bt) : 1;
+        }
+        __syncthreads();
+        // ---- serial steps, operands from LDS ----
+        for (int t = 0; t < tc; ++t) {
+            if (!on_s[t]) continue;                 // masked step: state untouched
+            const float4 k4 = *reinterpret_cast<const float4*>(&k_s[t][c4]);
+            float4 g4;
+            if (VEC_G) g4 = *reinterpret_cast<const float4*>(&g_s[t][c4]);
+            else { const float gs = g_s[0][t]; g4 = make_float4(gs, gs, gs, gs); }
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+                const float d = d_s[t][rsub + RPP * i];
+                s[i].x = requant<StateT>(fmaf(k4.x, d, s[i].x * g4.x));
+                s[i].y = requant<StateT>(fmaf(k4.y, d, s[i].y * g4.y));
+                s[i].z = requant<StateT>(fmaf(k4.z, d, s[i].z * g4.z));
+                s[i].w = requant<StateT>(fmaf(k4.w, d, s[i].w * g4.w));
+            }
+        }
+    }
+
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+        const int r = row0 + rsub + RPP * i;
+        if (r < A.Dv) store4(s_out + (size_t)r * DK + c4, s[i]);
+    }
+}
+
+template <typename StateT, bool VEC_G, int DK>
+static int launch_replay_nr(hipStream_t st, const ReplayBatch& P, const ReplayArgs& A, int B, int n_layers) {
+    constexpr int RPP = kThreads / (DK / 4);
+    // Fewer, fatter workgroups once the grid already covers the chip several times over.
+    const long wg1 = (long)((A.Dv + RPP - 1) / RPP) * B * A.Hv * n_layers;
+    const int cus = num_compute_units();
+    if (wg1 >= 16L * cus && A.Dv >= RPP * 4) {
+        dim3 grid((A.Dv + RPP * 4 - 1) / (RPP * 4), B * A.Hv, n_layers);
+        hipLaunchKernelGGL((tape_replay_kernel<StateT, VEC_G, DK, 4>), grid, dim3(kThreads), 0, st, P, A);
+    } else {
+        dim3 grid((A.Dv + RPP - 1) / RPP, B * A.Hv, n_layers);
+        hipLaunchKernelGGL((tape_replay_kernel<StateT, VEC_G, DK, 1>), grid, dim3(kThreads), 0, st, P, A);
+    }
+    DFLASH_HIP_TRY(hipGetLastError());
+    return DFLASH_OK;
+}
+
+template <typename StateT>
+static int launch_replay_state(hipStream_t st, const ReplayBatch& P, const ReplayArgs& A, int B, int n_layers,
+                               int g_ndim, int Dk) {
+    const bool vec = g_ndim == 4;
+#define DFLASH_REPLAY_CASE(DKV)                                                              \
+    case DKV:                                                                                \
+        return vec ? launch_replay_nr<StateT, true, DKV>(st, P, A, B, n_layers)              \
+                   : launch_replay_nr<StateT, false, DKV>(st, P, A, B, n_layers);
+    switch (Dk) {
+        DFLASH_REPLAY_CASE(32)
+        DFLASH_REPLAY_CASE(64)
+        DFLASH_REPLAY_CASE(128)
+        DFLASH_REPLAY_CASE(256)
+        default: break;
+    }
+#undef DFLASH_REPLAY_CASE
+    set_error("tape replay: Dk=%d is not one of 32, 64, 128, 256", Dk);
+    return DFLASH_UNSUPPORTED;
+}
+
+static int replay_common(hipStream_t st, int n_layers, const void* const* tape, int tape_dtype,
+                         const void* const* k, const void* const* g, int in_dtype, int g_ndim,
+                         const void* const* state_in, void* const* state_out, int state_dtype,
+                         const void* mask, int mask_dtype, int steps, const int32_t* steps_dev, int skip_if_full,
+                         int B, int T_tape, int Hk, int Hv, int Dk, int Dv) {
+    int rc = ensure_init();
+    if (rc) return rc;
+    DFLASH_REQUIRE(n_layers >= 1 && n_layers <= DFLASH_MAX_BATCHED_LAYERS, "tape replay: n_layers=%d out of range", n_layers);
+    DFLASH_REQUIRE(B > 0 && T_tape >= 0 && Hk > 0 && Hv > 0 && Dk > 0 && Dv > 0, "tape replay: non-positive dimension");
+    DFLASH_REQUIRE(Hv % Hk == 0, "tape replay: Hv=%d is not a multiple of Hk=%d", Hv, Hk);
+    DFLASH_REQUIRE(g_ndim == 3 || g_ndim == 4, "tape replay: g_ndim must be 3 or 4");
+    DFLASH_REQUIRE(steps >= 0 && steps <= T_tape, "tape replay: steps=%d outside [0, T=%d]", steps, T_tape);
+    DFLASH_REQUIRE((long)B * Hv <= 65535, "tape replay: B*Hv too large for one launch");
+    DFLASH_SUPPORTED(in_dtype == DFLASH_F32 || in_dtype == DFLASH_BF16 || in_dtype == DFLASH_F16, "tape replay: bad in_dtype %d", in_dtype);
+    DFLASH_SUPPORTED(tape_dtype == DFLASH_F32 || tape_dtype == in_dtype, "tape replay: tape dtype must be f32 or the input dtype");
+    DFLASH_SUPPORTED(state_dtype == DFLASH_F32 || state_dtype == in_dtype, "tape replay: state dtype must be f32 or the input dtype");
+    if (mask) DFLASH_REQUIRE(mask_dtype >= DFLASH_F32 && mask_dtype <= DFLASH_U8, "tape replay: bad mask dtype");
+
+    ReplayBatch P;
+    for (int l = 0; l < n_layers; ++l) {
+        DFLASH_REQUIRE(state_in[l] && state_out[l], "tape replay: null state pointer (layer %d)", l);
+        DFLASH_REQUIRE(state_in[l] != state_out[l], "tape replay: state_in aliases state_out (layer %d)", l);
+        DFLASH_REQUIRE(T_tape == 0 || (tape[l] && k[l] && g[l]), "tape replay: null input pointer (layer %d)", l);
+        P.tape[l] = tape[l]; P.k[l] = k[l]; P.g[l] = g[l];
+        P.state_in[l] = state_in[l]; P.state_out[l] = state_out[l];
+    }
+    ReplayArgs A;
+    A.mask = mask; A.steps_dev = steps_dev; A.mask_dtype = mask_dtype; A.tape_dtype = tape_dtype;
+    A.in_dtype = in_dtype; A.steps = steps; A.skip_if_full = skip_if_full;
+    A.T_tape = T_tape; A.Hk = Hk; A.Hv = Hv; A.Dv = Dv;
+
+    switch (state_dtype) {
+        case DFLASH_F32: return launch_replay_state<float>(st, P, A, B, n_layers, g_ndim, Dk);
+        case DFLASH_BF16: return launch_replay_state<bf16_t>(st, P, A, B, n_layers, g_ndim, Dk);
+        default: return launch_replay_state<f16_t>(st, P, A, B, n_layers, g_ndim, Dk);
+    }
+}
+
+// ===========================================================================
+// Gated delta forward with tape
+// ===========================================================================
+
+struct GdnArgs {
+    const void *q, *k, *v, *g, *beta, *mask;
+    const void* state_in;
+    void* state_out;
+    void* y;
+    float* tape;
+    int in_dtype, mask_dtype;
+    int T, Hk, Hv, Dv;
+};
+
+constexpr int kGdnChunk = 16;  // steps staged in LDS at a time
+
+// LPR lanes share one state row; each keeps DK/LPR channels as float4 pieces
+// interleaved across the group (piece c of lane j covers channels
+// c*4*LPR + 4j .. +3) so that state loads and stores are fully coalesced.
+// The two row dot products (S'k for the innovation, S'q for the read-out) are
+// reduced together with DPP adds inside the 16-lane row; the read-out uses
+//   y = (S' + delta (x) k) q = S'q + delta * (k.q),
+// so the second reduction does not wait for delta.
+// Grid: x = Dv tiles of ROWS = 256/LPR rows, y = b*Hv + hv.
+template <typename StateT, bool VEC_G, int DK, int LPR>
+__global__ __launch_bounds__(kThreads) void gated_delta_tape_kernel(GdnArgs A) {
+    constexpr int ROWS = kThreads / LPR;
+    constexpr int CH = DK / (4 * LPR);
+    constexpr int TC = kGdnChunk;
+    static_assert(CH >= 1, "row slice must hold at least one float4");
+
+    __shared__ float q_s[TC][DK];
+    __shared__ float k_s[TC][DK];
+    __shared__ float g_s[VEC_G ? TC : 1][VEC_G ? DK : TC];
+    __shared__ float v_s[TC][ROWS];
+    __shared__ float y_s[TC][ROWS];
+    __shared__ float t_s[TC][ROWS];
+    __shared__ float beta_s[TC];
+    __shared__ float kq_s[TC];
+    __shared__ int on_s[TC];
+
+    const int bh = blockIdx.y;
+    const int b = bh / A.Hv, hv = bh % A.Hv;
+    const int hk = hv / (A.Hv / A.Hk);
+    const int row0 = blockIdx.x * ROWS;
+    const int tid = threadIdx.x;
+    const int j = tid % LPR;
+    const int rloc = tid / LPR;
+    const int row = row0 + rloc;
+    const bool row_ok = row < A.Dv;
+
+    const StateT* s_in = reinterpret_cast<const StateT*>(A.state_in) + ((size_t)bh * A.Dv + (row_ok ? row : 0)) * DK;
+    StateT* s_out = reinterpret_cast<StateT*>(A.state_out) + ((size_t)bh * A.Dv + (row_ok ? row : 0)) * DK;
+
+    float4 s[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) s[c] = load4(s_in + c * 4 * LPR + 4 * j);
+
+    for (int t0 = 0; t0 < A.T; t0 += TC) {
+        const int tc = (A.T - t0) < TC ? (A.T - t0) : TC;
+        if (t0) __syncthreads();
+        // ---- stage operands of this chunk as float ----
+        for (int i = tid; i < tc * (DK / 4); i += kThreads) {
+            const int t = i / (DK / 4), c = (i % (DK / 4)) * 4;
+            const size_t bt = (size_t)b * A.T + t0 + t;
+            store4(&q_s[t][c], load4_rt(A.q, A.in_dtype, (bt * A.Hk + hk) * DK + c));
+            store4(&k_s[t][c], load4_rt(A.k, A.in_dtype, (bt * A.Hk + hk) * DK + c));
+            if (VEC_G) store4(&g_s[t][c], load4_rt(A.g, A.in_dtype, (bt * A.Hv + hv) * DK + c));
+        }
+        for (int i = tid; i < tc * ROWS; i += kThreads) {
+            const int t = i / ROWS, r = i % ROWS;
+            const size_t bt = (size_t)b * A.T + t0 + t;
+            v_s[t][r] = (row0 + r) < A.Dv ? load1_rt(A.v, A.in_dtype, (bt * A.Hv + hv) * A.Dv + row0 + r) : 0.f;
+        }
+        if (tid < tc) {
+            const size_t bt = (size_t)b * A.T + t0 + tid;
+            if (!VEC_G) g_s[0][tid] = load1_rt(A.g, A.in_dtype, bt * A.Hv + hv);
+            beta_s[tid] = load1_rt(A.beta, A.in_dtype, bt * A.Hv + hv);
+            on_s[tid] = A.mask ? (int)mask_on(A.mask, A.mask_dtype, (int)bt) : 1;
+        }
+        __syncthreads();
+        // k.q per step: 16 lanes per step, 16 steps per pass of the workgroup
+        for (int t = tid / 16; t < tc; t += kThreads / 16) {
+            float acc = 0.f;
+            for (int d = tid % 16; d < DK; d += 16) acc = fmaf(k_s[t][d], q_s[t][d], acc);
+            acc = group_sum<16>(acc);
+            if (tid % 16 == 0) kq_s[t] = acc;
+        }
+        __syncthreads();
+
+        // ---- serial steps ----
+        for (int t = 0; t < tc; ++t) {
+            float yv = 0.f, delta = 0.f;
+            if (on_s[t]) {                            // uniform across the workgroup
+                float sk = 0.f, sq = 0.f;
+#pragma unroll
+                for (int c = 0; c < CH; ++c) {
+                    const int d = c * 4 * LPR + 4 * j;
+                    const float4 k4 = *reinterpret_cast<const float4*>(&k_s[t][d]);
+                    const float4 q4 = *reinterpret_cast<const float4*>(&q_s[t][d]);
+                    float4 g4;
+                    if (VEC_G) g4 = *reinterpret_cast<const float4*>(&g_s[t][d]);
+                    else { const float gs = g_s[0][t]; g4 = make_float4(gs, gs, gs, gs); }
+                    s[c].x *= g4.x; s[c].y *= g4.y; s[c].z *= g4.z; s[c].w *= g4.w;
+                    sk = fmaf(s[c].x, k4.x, sk); sk = fmaf(s[c].y, k4.y, sk);
+                    sk = fmaf(s[c].z, k4.z, sk); sk = fmaf(s[c].w, k4.w, sk);
+                    sq = fmaf(s[c].x, q4.x, sq); sq = fmaf(s[c].y, q4.y, sq);
+                    sq = fmaf(s[c].z, q4.z, sq); sq = fmaf(s[c].w, q4.w, sq);
+                }
+                sk = group_sum<LPR>(sk);
+                sq = group_sum<LPR>(sq);
+                delta = (v_s[t][rloc] - sk) * beta_s[t];
+                yv = fmaf(delta, kq_s[t], sq);
+#pragma unroll
+                for (int c = 0; c < CH; ++c) {
+                    const int d = c * 4 * LPR + 4 * j;
+                    const float4 k4 = *reinterpret_cast<const float4*>(&k_s[t][d]);
+                    s[c].x = requant<StateT>(fmaf(k4.x, delta, s[c].x));
+                    s[c].y = requant<StateT>(fmaf(k4.y, delta, s[c].y));
+                    s[c].z = requant<StateT>(fmaf(k4.z, delta, s[c].z));
+                    s[c].w = requant<StateT>(fmaf(k4.w, delta, s[c].w));
+                }
+            }
+            if (j == 0) { y_s[t][rloc] = yv; t_s[t][rloc] = delta; }
+        }
+        __syncthreads();
+        // ---- write this chunk's y and tape rows ----
+        for (int i = tid; i < tc * ROWS; i += kThreads) {
+            const int t = i / ROWS, r = i % ROWS;
+            if (row0 + r < A.Dv) {
+                const size_t o = (((size_t)b * A.T + t0 + t) * A.Hv + hv) * A.Dv + row0 + r;
+                store1_rt(A.y, A.in_dtype, o, y_s[t][r]);
+                A.tape[o] = t_s[t][r];
+            }
+        }
+    }
+
+    if (row_ok) {
+#pragma unroll
+        for (int c = 0; c < CH; ++c) store4(s_out + c * 4 * LPR + 4 * j, s[c]);
+    }
+}
+
+template <typename StateT>
+static int launch_gdn_state(hipStream_t st, const GdnArgs& A, int B, int g_ndim, int Dk) {
+    const bool vec = g_ndim == 4;
+#define DFLASH_GDN_CASE(DKV, LPRV)                                                                     \
+    case DKV: {                                                                                        \
+        dim3 grid((A.Dv + (kThreads / LPRV) - 1) / (kThreads / LPRV), B * A.Hv);                       \
+        if (vec) hipLaunchKernelGGL((gated_delta_tape_kernel<StateT, true, DKV, LPRV>), grid, dim3(kThreads), 0, st, A); \
+        else hipLaunchKernelGGL((gated_delta_tape_kernel<StateT, false, DKV, LPRV>), grid, dim3(kThreads), 0, st, A);    \
+        DFLASH_HIP_TRY(hipGetLastError());                                                             \
+        return DFLASH_OK;                                                                              \
+    }
+    switch (Dk) {
+        DFLASH_GDN_CASE(32, 8)
+        DFLASH_GDN_CASE(64, 16)
+        DFLASH_GDN_CASE(128, 16)
+        DFLASH_GDN_CASE(256, 16)
+        default: break;
+    }
+#undef DFLASH_GDN_CASE
+    set_error("gated delta: Dk=%d is not one of 32, 64, 128, 256", Dk);
+    return DFLASH_UNSUPPORTED;
+}
+
+}  // namespace dflash
+
+using namespace dflash;
+
+extern "C" int dflash_tape_replay(void* stream, const void* tape, int tape_dtype, const void* k, const void* g,
+                                  int in_dtype, int g_ndim, const void* state_in, void* state_out, int state_dtype,
+                                  const void* mask, int mask_dtype, int B, int T, int Hk, int Hv, int Dk, int Dv) {
+    const void* tp[1] = {tape};
+    const void* kp[1] = {k};
+    const void* gp[1] = {g};
+    const void* si[1] = {state_in};
+    void* so[1] = {state_out};
+    return replay_common((hipStream_t)stream, 1, tp, tape_dtype, kp, gp, in_dtype, g_ndim, si, so, state_dtype,
+                         mask, mask_dtype, T, nullptr, 0, B, T, Hk, Hv, Dk, Dv);
+}
+
+extern "C" int dflash_tape_replay_batched(void* stream, int n_layers, const void* const* tape, int tape_dtype,
+                                          const void* const* k, const void* const* g, int in_dtype, int g_ndim,
+                                          const void* const* state_in, void* const* state_out, int state_dtype,
+                                          int steps, const int32_t* steps_dev, int skip_if_full, int B, int T_tape,
+                                          int Hk, int Hv, int Dk, int Dv) {
+    DFLASH_REQUIRE(tape && k && g && state_in && state_out, "tape replay (batched): null pointer array");
+    return replay_common((hipStream_t)stream, n_layers, tape, tape_dtype, k, g, in_dtype, g_ndim, state_in, state_out,
+                         state_dtype, nullptr, 0, steps, steps_dev, skip_if_full, B, T_tape, Hk, Hv, Dk, Dv);
+}
+
+extern "C" int dflash_gated_delta_tape(void* stream, const void* q, const void* k, const void* v, const void* g,
+                                       int g_ndim, const void* beta, int in_dtype, const void* state_in,
+                                       void* state_out, int state_dtype, void* y, float* tape_out, const void* mask,
+                                       int mask_dtype, int B, int T, int Hk, int Hv, int Dk, int Dv) {
+    int rc = ensure_init();
+    if (rc) return rc;
+    DFLASH_REQUIRE(B > 0 && T >= 0 && Hk > 0 && Hv > 0 && Dk > 0 && Dv > 0, "gated delta: non-positive dimension");
+    DFLASH_REQUIRE(Hv % Hk == 0, "gated delta: Hv=%d is not a multiple of Hk=%d", Hv, Hk);
+    DFLASH_REQUIRE(g_ndim == 3 || g_ndim == 4, "gated delta: g_ndim must be 3 or 4");
+    DFLASH_REQUIRE(state_in && state_out, "gated delta: null state pointer");
+    DFLASH_REQUIRE(state_in != state_out, "gated delta: state_in aliases state_out");
+    DFLASH_REQUIRE(T == 0 || (q && k && v && g && beta && y && tape_out), "gated delta: null pointer");
+    DFLASH_REQUIRE((long)B * Hv <= 65535, "gated delta: B*Hv too large for one launch");
+    DFLASH_SUPPORTED(in_dtype == DFLASH_F32 || in_dtype == DFLASH_BF16 || in_dtype == DFLASH_F16, "gated delta: bad in_dtype %d", in_dtype);
+    DFLASH_SUPPORTED(state_dtype == DFLASH_F32 || state_dtype == in_dtype, "gated delta: state dtype must be f32 or the input dtype");
+    if (mask) DFLASH_REQUIRE(mask_dtype >= DFLASH_F32 && mask_dtype <= DFLASH_U8, "gated delta: bad mask dtype");
+
+    GdnArgs A;
+    A.q = q; A.k = k; A.v = v; A.g = g; A.beta = beta; A.mask = mask;
+    A.state_in = state_in; A.state_out = state_out; A.y = y; A.tape = tape_out;
+    A.in_dtype = in_dtype; A.mask_dtype = mask_dtype; A.T = T; A.Hk = Hk; A.Hv = Hv; A.Dv = Dv;
+    switch (state_dtype) {
+        case DFLASH_F32: return launch_gdn_state<float>((hipStream_t)stream, A, B, g_ndim, Dk);
+        case DFLASH_BF16: return launch_gdn_state<bf16_t>((hipStream_t)stream, A, B, g_ndim, Dk);
+        default: return launch_gdn_state<f16_t>((hipStream_t)stream, A, B, g_ndim, Dk);
+    }
+}

@@ -1,0 +1,215 @@
+"""Host-side mirror of ``DFlashKernels`` (Sources/DFlash/DFlashKernels.swift) and
+``DFlashKernelProvider`` / ``DFlashKernelRegistry``
+(Sources/DFlash/DFlashKernelProvider.swift) over the HIP C ABI.
+
+Same entry-point names, argument meaning and error behaviour as the reference:
+each call is functional (inputs untouched, freshly allocated outputs).  torch is
+used only to own device memory and to name the current stream; every result is
+computed by libdflash_hip.so.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import DFlashError, DFlashUnsupported  # noqa: F401  (re-exported)
+
+_DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16,
+       torch.uint8: _lib.U8, torch.bool: _lib.U8}
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise DFlashUnsupported(f"dtype {t.dtype} is not supported") from None
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev(*ts: Optional[torch.Tensor]) -> None:
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise DFlashError("DFlash kernels run on the GPU only: got a CPU tensor (there is no CPU path)")
+
+
+def _ptr_array(ts: Sequence[torch.Tensor]):
+    arr = (C.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+    return C.cast(arr, _lib.vpp), arr
+
+
+class DFlashKernels:
+    """Static entry points, named as in the reference."""
+
+    shared: "DFlashKernelsInstance"
+
+    # -- tape replay ---------------------------------------------------------
+    @staticmethod
+    def tape_replay_kernel(tape: torch.Tensor, k: torch.Tensor, g: torch.Tensor, state: torch.Tensor,
+                           mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``tapeReplayKernel(tape:k:g:state:mask:)`` (DFlashKernels.swift:252-301).
+
+        tape [B,T,Hv,Dv], k [B,T,Hk,Dk], g [B,T,Hv] or [B,T,Hv,Dk], state
+        [B,Hv,Dv,Dk], mask [B,T]; returns the replayed state (same dtype as ``state``).
+        """
+        _dev(tape, k, g, state, mask)
+        tape, k, g, state = (t.contiguous() for t in (tape, k, g, state))
+        if g.dtype != k.dtype:
+            g = g.to(k.dtype)
+        mask = None if mask is None else mask.contiguous()
+        B, T, Hk, Dk = k.shape
+        Hv, Dv = tape.shape[2], tape.shape[3]
+        out = torch.empty_like(state)
+        rc = _lib.load().dflash_tape_replay(
+            _stream(), _ptr(tape), _code(tape), _ptr(k), _ptr(g), _code(k), g.dim(),
+            _ptr(state), _ptr(out), _code(state), _ptr(mask), _code(mask) if mask is not None else 0,
+            B, T, Hk, Hv, Dk, Dv)
+        _lib.check(rc, "tape_replay_kernel")
+        return out
+
+    @staticmethod
+    def tape_replay_batched(tapes: Sequence[torch.Tensor], ks: Sequence[torch.Tensor], gs: Sequence[torch.Tensor],
+                            states_in: Sequence[torch.Tensor], states_out: Sequence[torch.Tensor], steps: int,
+                            steps_dev: Optional[torch.Tensor] = None, skip_if_full: bool = False) -> None:
+        """One launch for the per-cache replays that
+        ``restoreTargetCacheAfterAcceptance`` issues one by one
+        (DFlashRuntime.swift:197-205).  All layers share shapes; results are written
+        into ``states_out``."""
+        _dev(*tapes, *ks, *gs, *states_in, *states_out, steps_dev)
+        n = len(tapes)
+        B, T, Hk, Dk = ks[0].shape
+        Hv, Dv = tapes[0].shape[2], tapes[0].shape[3]
+        for seq in (tapes, ks, gs, states_in, states_out):
+            if len(seq) != n or any(not t.is_contiguous() for t in seq):
+                raise DFlashError("tape_replay_batched: ragged or non-contiguous layer list")
+        pt, _k1 = _ptr_array(tapes)
+        pk, _k2 = _ptr_array(ks)
+        pg, _k3 = _ptr_array(gs)
+        pi, _k4 = _ptr_array(states_in)
+        po, _k5 = _ptr_array(states_out)
+        rc = _lib.load().dflash_tape_replay_batched(
+            _stream(), n, pt, _code(tapes[0]), pk, pg, _code(ks[0]), gs[0].dim(), pi, po, _code(states_in[0]),
+            int(steps), _ptr(steps_dev), int(bool(skip_if_full)), B, T, Hk, Hv, Dk, Dv)
+        _lib.check(rc, "tape_replay_batched")
+
+    # -- gated delta with tape -------------------------------------------------
+    @staticmethod
+    def gated_delta_kernel_with_tape(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor,
+                                     beta: torch.Tensor, state: torch.Tensor,
+                                     mask: Optional[torch.Tensor] = None
+                                     ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """``gatedDeltaKernelWithTape(q:k:v:g:beta:state:mask:)`` (DFlashKernels.swift:316-367).
+
+        Returns (y [B,T,Hv,Dv] in q's dtype, new state in ``state``'s dtype,
+        innovation tape [B,T,Hv,Dv] float32)."""
+        _dev(q, k, v, g, beta, state, mask)
+        q, k, v, g, beta, state = (t.contiguous() for t in (q, k, v, g, beta, state))
+        for name, t in (("k", k), ("v", v), ("g", g), ("beta", beta)):
+            if t.dtype != q.dtype:
+                raise DFlashUnsupported(f"gated_delta_kernel_with_tape: {name} dtype {t.dtype} differs from q's {q.dtype}")
+        mask = None if mask is None else mask.contiguous()
+        B, T, Hk, Dk = k.shape
+        Hv, Dv = v.shape[2], v.shape[3]
+        y = torch.empty((B, T, Hv, Dv), dtype=q.dtype, device=q.device)
+        tape = torch.empty((B, T, Hv, Dv), dtype=torch.float32, device=q.device)
+        out = torch.empty_like(state)
+        rc = _lib.load().dflash_gated_delta_tape(
+            _stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(g), g.dim(), _ptr(beta), _code(q),
+            _ptr(state), _ptr(out), _code(state), _ptr(y), _ptr(tape),
+            _ptr(mask), _code(mask) if mask is not None else 0, B, T, Hk, Hv, Dk, Dv)
+        _lib.check(rc, "gated_delta_kernel_with_tape")
+        return y, out, tape
+
+    # -- block-causal SDPA -------------------------------------------------------
+    @staticmethod
+    def sdpa_workspace_bytes(B: int, Hq: int, Hk: int, M: int, N: int, D: int) -> int:
+        return int(_lib.load().dflash_sdpa_workspace_bytes(B, Hq, Hk, M, N, D))
+
+    @staticmethod
+    def batched_sdpa_2pass(queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, scale: float,
+                           mask: Optional[torch.Tensor] = None, *, return_lse: bool = False,
+                           kv_len: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None):
+        """``batchedSDPA2Pass(queries:keys:values:scale:mask:)`` (DFlashKernels.swift:737-815).
+
+        queries [B,Hq,16,D]; keys/values [B,Hk,N,D] with N including the 16 block
+        tokens (a view into a larger cache is fine as long as the last dimension is
+        contiguous and rows are D apart).  Returns None where the reference returns
+        nil (unsupported shape/dtype).  ``return_lse`` additionally returns the
+        float32 logsumexp [B,Hq,16]; ``kv_len`` (int32 [B] on the device) gives
+        per-sequence key counts for ragged batches."""
+        if queries.dim() != 4 or keys.dim() != 4 or values.dim() != 4:
+            return None
+        if mask is not None:
+            return None   # additive masks are not covered by the HIP kernel
+        _dev(queries, keys, values, kv_len, workspace)
+        B, Hq, M, D = queries.shape
+        Hk, N = keys.shape[1], keys.shape[2]
+        if values.shape != keys.shape or values.shape[3] != D or keys.dtype != queries.dtype or values.dtype != queries.dtype:
+            return None
+        queries = queries.contiguous()
+        if keys.stride(3) != 1 or keys.stride(2) != D or keys.stride() != values.stride():
+            keys, values = keys.contiguous(), values.contiguous()
+        lib = _lib.load()
+        need = int(lib.dflash_sdpa_workspace_bytes(B, Hq, Hk, M, N, D))
+        if need == 0:
+            return None
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=queries.device)
+        out = torch.empty_like(queries)
+        lse = torch.empty((B, Hq, M), dtype=torch.float32, device=queries.device) if return_lse else None
+        try:
+            code = _code(queries)
+        except DFlashUnsupported:
+            return None
+        rc = lib.dflash_sdpa_block_causal(
+            _stream(), _ptr(queries), _ptr(keys), _ptr(values), _ptr(out), _ptr(lse), code, float(scale),
+            B, Hq, Hk, M, N, D, keys.stride(0), keys.stride(1), _ptr(kv_len), _ptr(workspace),
+            workspace.numel() * workspace.element_size())
+        if rc == _lib.UNSUPPORTED:
+            return None
+        _lib.check(rc, "batched_sdpa_2pass")
+        return (out, lse) if return_lse else out
+
+    @staticmethod
+    def sdpa_fallback(queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, scale: float,
+                      mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``sdpaFallback`` (DFlashKernels.swift:818-828) delegates to the array library's
+        general attention.  This package ships only the verify-block kernel, so shapes
+        it does not cover are an error here instead of a silent second path."""
+        out = DFlashKernels.batched_sdpa_2pass(queries, keys, values, scale, mask)
+        if out is None:
+            raise DFlashUnsupported("sdpa_fallback: shape/dtype not covered by the verify-block attention kernel")
+        return out
+
+
+class DFlashKernelProvider:
+    """``protocol DFlashKernelProvider`` (DFlashKernelProvider.swift:8-14)."""
+
+    def gated_delta_kernel_with_tape(self, q, k, v, g, beta, state, mask):  # pragma: no cover - protocol
+        raise NotImplementedError
+
+
+class DFlashKernelsInstance(DFlashKernelProvider):
+    """``DFlashKernelsInstance`` (DFlashKernels.swift:832-843)."""
+
+    def gated_delta_kernel_with_tape(self, q, k, v, g, beta, state, mask=None):
+        return DFlashKernels.gated_delta_kernel_with_tape(q, k, v, g, beta, state, mask)
+
+
+DFlashKernels.shared = DFlashKernelsInstance()
+
+
+class DFlashKernelRegistry:
+    """``DFlashKernelRegistry.provider`` (DFlashKernelProvider.swift:17-19)."""
+
+    provider: Optional[DFlashKernelProvider] = None

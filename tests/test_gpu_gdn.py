@@ -1,0 +1,233 @@
+"""GPU parity: GatedDelta forward-with-tape and tape replay (HIP, through the C ABI)
+against the CPU oracle on the same seeded inputs.
+
+Bars (BASELINE north_star): fp32 recurrent state rtol 1e-4 (atol 1e-6 for entries
+near zero); bf16/f16 outputs 2e-2 abs/rel; the fp32 tape is held to the state's bar.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import dflash_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TORCH_DT = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+STATE_TOL = dict(rtol=1e-4, atol=1e-6)
+LOWP_TOL = dict(rtol=2e-2, atol=2e-2)
+
+
+def dev(a, dt="f32"):
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda", TORCH_DT[dt])
+
+
+def host(t):
+    return t.detach().float().cpu().numpy()
+
+
+def make_mask(seed, B, T):
+    rng = np.random.default_rng(seed)
+    m = (rng.random((B, T)) < 0.6).astype(np.float32)
+    m[:, 0] = 1.0
+    return m
+
+
+def run_forward(K, d, in_dt, state_dt, mask=None, mask_dt="f32"):
+    args = [dev(d[n], in_dt) for n in ("q", "k", "v", "g", "beta")]
+    state = dev(d["state"], state_dt)
+    m = None if mask is None else (torch.from_numpy(mask).to("cuda").to(torch.uint8) if mask_dt == "u8"
+                                   else dev(mask, mask_dt))
+    y, s, tape = K.gated_delta_kernel_with_tape(*args, state, m)
+    torch.cuda.synchronize()
+    return y, s, tape
+
+
+# (name, B, T, Hk, Hv, Dk, Dv)
+SHAPES = [
+    ("cfg0", 1, 8, 4, 8, 64, 64),
+    ("cfg1", 1, 16, 16, 32, 128, 128),
+    ("ragged_dv", 2, 5, 2, 6, 128, 40),
+    ("dk32", 1, 7, 2, 4, 32, 24),
+    ("dk256", 1, 6, 1, 2, 256, 64),
+    ("long_T", 1, 40, 2, 4, 64, 32),
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=[s[0] for s in SHAPES])
+@pytest.mark.parametrize("vec", [False, True], ids=["scalar_g", "vec_g"])
+@pytest.mark.parametrize("in_dt", ["f32", "bf16"])
+def test_forward_matches_oracle(gpu_lib, shape, vec, in_dt):
+    from swiftlm_amd import DFlashKernels as K
+
+    name, B, T, Hk, Hv, Dk, Dv = shape
+    d = O.make_gdn_inputs(100 + len(name), B, T, Hk, Hv, Dk, Dv, in_dtype=in_dt, vec_gate=vec)
+    y, s, tape = run_forward(K, d, in_dt, "f32")
+    yw, sw, tw = O.gated_delta_ops_with_tape(d["q"], d["k"], d["v"], d["g"], d["beta"], d["state"], dtype=np.float64)
+    assert y.dtype == TORCH_DT[in_dt] and s.dtype == torch.float32 and tape.dtype == torch.float32
+    np.testing.assert_allclose(host(s), sw, **STATE_TOL)
+    np.testing.assert_allclose(host(tape), tw, rtol=1e-4, atol=1e-5)
+    if in_dt == "f32":
+        np.testing.assert_allclose(host(y), yw, rtol=1e-4, atol=1e-5)
+    else:
+        np.testing.assert_allclose(host(y), yw, **LOWP_TOL)
+
+
+@pytest.mark.parametrize("vec", [False, True], ids=["scalar_g", "vec_g"])
+@pytest.mark.parametrize("mask_dt", ["f32", "bf16", "u8"])
+def test_forward_masked(gpu_lib, vec, mask_dt):
+    from swiftlm_amd import DFlashKernels as K
+
+    B, T, Hk, Hv, Dk, Dv = 2, 12, 2, 4, 128, 48
+    d = O.make_gdn_inputs(7, B, T, Hk, Hv, Dk, Dv, in_dtype="bf16", vec_gate=vec)
+    mask = make_mask(8, B, T)
+    y, s, tape = run_forward(K, d, "bf16", "f32", mask, mask_dt)
+    yw, sw, tw = O.gated_delta_ops_with_tape(d["q"], d["k"], d["v"], d["g"], d["beta"], d["state"], mask,
+                                             dtype=np.float64)
+    np.testing.assert_allclose(host(s), sw, **STATE_TOL)
+    np.testing.assert_allclose(host(tape), tw, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(host(y), yw, **LOWP_TOL)
+    off = mask < 0.5
+    assert np.all(host(y)[off] == 0) and np.all(host(tape)[off] == 0)     # exact zeros on masked steps
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+def test_forward_low_precision_state_requantises_each_step(gpu_lib, dt):
+    """State stored in the input type: rounded after every step like the Metal kernel
+    (DFlashKernels.swift:183-186)."""
+    from swiftlm_amd import DFlashKernels as K
+
+    B, T, Hk, Hv, Dk, Dv = 1, 8, 2, 4, 128, 32
+    d = O.make_gdn_inputs(9, B, T, Hk, Hv, Dk, Dv, in_dtype=dt)
+    d["state"] = O.quantize(d["state"], dt)
+    y, s, tape = run_forward(K, d, dt, dt)
+    assert s.dtype == TORCH_DT[dt]
+    yw, sw, tw = O.gated_delta_ops_with_tape(d["q"], d["k"], d["v"], d["g"], d["beta"], d["state"], requant=dt)
+    np.testing.assert_allclose(host(s), sw, **LOWP_TOL)
+    np.testing.assert_allclose(host(y), yw, **LOWP_TOL)
+    np.testing.assert_allclose(host(tape), tw, **LOWP_TOL)
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=[s[0] for s in SHAPES])
+@pytest.mark.parametrize("vec", [False, True], ids=["scalar_g", "vec_g"])
+def test_replay_matches_oracle_for_every_prefix(gpu_lib, shape, vec):
+    from swiftlm_amd import DFlashKernels as K
+
+    name, B, T, Hk, Hv, Dk, Dv = shape
+    in_dt = "f32" if name == "cfg0" else "bf16"
+    d = O.make_gdn_inputs(200 + len(name), B, T, Hk, Hv, Dk, Dv, in_dtype=in_dt, vec_gate=vec)
+    rng = np.random.default_rng(3)
+    tape = rng.standard_normal((B, T, Hv, Dv)).astype(np.float32)
+    tape_d, k_d, g_d, s_d = dev(tape), dev(d["k"], in_dt), dev(d["g"], in_dt), dev(d["state"])
+    steps = sorted(set([1, 2, T // 2, T - 1, T]) - {0})
+    for n in steps:                                    # the caller slices the accepted prefix
+        out = K.tape_replay_kernel(tape_d[:, :n], k_d[:, :n], g_d[:, :n], s_d)
+        torch.cuda.synchronize()
+        want = O.tape_replay_ops(tape[:, :n], d["k"][:, :n], d["g"][:, :n], d["state"], dtype=np.float64)
+        np.testing.assert_allclose(host(out), want, **STATE_TOL, err_msg=f"n={n}")
+    # T == 0 returns the input state
+    out = K.tape_replay_kernel(tape_d[:, :0], k_d[:, :0], g_d[:, :0], s_d)
+    assert torch.equal(out, s_d)
+
+
+def test_replay_masked_and_bf16_tape(gpu_lib):
+    from swiftlm_amd import DFlashKernels as K
+
+    B, T, Hk, Hv, Dk, Dv = 2, 16, 8, 16, 128, 128        # the reference bench's shape (DFlashKernelBench/main.swift:107)
+    d = O.make_gdn_inputs(11, B, T, Hk, Hv, Dk, Dv, in_dtype="bf16")
+    tape = O.round_to_bf16(np.random.default_rng(4).uniform(-0.1, 0.1, (B, T, Hv, Dv)).astype(np.float32))
+    mask = make_mask(12, B, T)
+    out = K.tape_replay_kernel(dev(tape, "bf16"), dev(d["k"], "bf16"), dev(d["g"], "bf16"), dev(d["state"]),
+                               dev(mask, "bf16"))
+    want = O.tape_replay_ops(tape, d["k"], d["g"], d["state"], mask, dtype=np.float64)
+    np.testing.assert_allclose(host(out), want, **STATE_TOL)
+    # all-zero mask: state untouched bit for bit
+    out = K.tape_replay_kernel(dev(tape, "bf16"), dev(d["k"], "bf16"), dev(d["g"], "bf16"), dev(d["state"]),
+                               dev(np.zeros_like(mask)))
+    assert np.array_equal(host(out), d["state"])
+
+
+def test_replay_low_precision_state(gpu_lib):
+    from swiftlm_amd import DFlashKernels as K
+
+    B, T, Hk, Hv, Dk, Dv = 1, 8, 8, 16, 128, 128
+    rng = np.random.default_rng(5)
+    u = lambda *s: O.round_to_bf16(rng.uniform(-0.1, 0.1, s).astype(np.float32))   # DFlashKernelBench inputs (main.swift:28-30)
+    tape, k, g, state = u(B, T, Hv, Dv), u(B, T, Hk, Dk), u(B, T, Hv), u(B, Hv, Dv, Dk)
+    out = K.tape_replay_kernel(dev(tape, "bf16"), dev(k, "bf16"), dev(g, "bf16"), dev(state, "bf16"))
+    assert out.dtype == torch.bfloat16
+    want = O.tape_replay_ops(tape, k, g, state, requant="bf16")
+    # the reference's own consistency bar for this kernel (tests/DFlash/DFlashProfiler.swift:239)
+    a, b = host(out).ravel(), want.ravel()
+    assert np.abs(a - b).max() < 0.01
+    assert a @ b / (np.linalg.norm(a) * np.linalg.norm(b)) > 0.999
+    np.testing.assert_allclose(a, b, **LOWP_TOL)
+
+
+def test_forward_tape_replays_to_forward_state_at_full_size(gpu_lib):
+    """Size-independent property at the Qwen3-Next shape: replaying the recorded tape
+    for n steps from the pre-verify state gives the state of a forward over n tokens."""
+    from swiftlm_amd import DFlashKernels as K
+
+    B, T, Hk, Hv, Dk, Dv = 1, 16, 16, 32, 128, 128
+    rng = np.random.default_rng(6)
+    for layer in range(4):
+        d = O.make_gdn_inputs(1000 + layer, B, T, Hk, Hv, Dk, Dv, in_dtype="bf16")
+        q, k, v, g, beta = (dev(d[n], "bf16") for n in ("q", "k", "v", "g", "beta"))
+        s0 = dev(d["state"])
+        y, s_full, tape = K.gated_delta_kernel_with_tape(q, k, v, g, beta, s0)
+        n = O.draw_accepted(rng, T, "geometric")
+        _, s_n, _ = K.gated_delta_kernel_with_tape(q[:, :n].contiguous(), k[:, :n].contiguous(),
+                                                   v[:, :n].contiguous(), g[:, :n].contiguous(),
+                                                   beta[:, :n].contiguous(), s0)
+        rep = K.tape_replay_kernel(tape[:, :n], k[:, :n], g[:, :n], s0)
+        np.testing.assert_allclose(host(rep), host(s_n), **STATE_TOL)
+        rep_full = K.tape_replay_kernel(tape, k, g, s0)
+        np.testing.assert_allclose(host(rep_full), host(s_full), **STATE_TOL)
+        assert torch.equal(s0, dev(d["state"]))             # inputs are never written
+
+
+def test_batched_replay_equals_per_layer_replay(gpu_lib):
+    from swiftlm_amd import DFlashKernels as K
+
+    B, T, Hk, Hv, Dk, Dv, L = 1, 16, 16, 32, 128, 128, 36
+    rng = np.random.default_rng(7)
+    tapes, ks, gs, sin = [], [], [], []
+    for layer in range(L):
+        d = O.make_gdn_inputs(2000 + layer, B, T, Hk, Hv, Dk, Dv, in_dtype="bf16")
+        tapes.append(dev(rng.standard_normal((B, T, Hv, Dv)).astype(np.float32)))
+        ks.append(dev(d["k"], "bf16")); gs.append(dev(d["g"], "bf16")); sin.append(dev(d["state"]))
+    for n in (1, 4, 16):
+        sout = [torch.full_like(s, float("nan")) for s in sin]
+        K.tape_replay_batched(tapes, ks, gs, sin, sout, steps=n)
+        torch.cuda.synchronize()
+        for layer in (0, 17, 35):
+            one = K.tape_replay_kernel(tapes[layer][:, :n], ks[layer][:, :n], gs[layer][:, :n], sin[layer])
+            assert torch.equal(sout[layer], one), f"layer {layer} n={n}"
+        want = O.tape_replay_ops(host(tapes[5])[:, :n], host(ks[5])[:, :n], host(gs[5])[:, :n], host(sin[5]),
+                                 dtype=np.float64)
+        np.testing.assert_allclose(host(sout[5]), want, **STATE_TOL)
+    # step count read on the device; a fully accepted block leaves state_out alone
+    steps_dev = torch.tensor([3], dtype=torch.int32, device="cuda")
+    sout = [torch.zeros_like(s) for s in sin]
+    K.tape_replay_batched(tapes, ks, gs, sin, sout, steps=0, steps_dev=steps_dev, skip_if_full=True)
+    assert torch.equal(sout[9], K.tape_replay_kernel(tapes[9][:, :3], ks[9][:, :3], gs[9][:, :3], sin[9]))
+    steps_dev.fill_(T)
+    marker = [torch.full_like(s, 7.0) for s in sin]
+    K.tape_replay_batched(tapes, ks, gs, sin, marker, steps=0, steps_dev=steps_dev, skip_if_full=True)
+    torch.cuda.synchronize()
+    assert all(bool((m == 7.0).all()) for m in marker)
+
+
+def test_unsupported_and_invalid_arguments(gpu_lib):
+    from swiftlm_amd import DFlashKernels as K, DFlashError, DFlashUnsupported
+
+    d = O.make_gdn_inputs(1, 1, 4, 2, 4, 48, 16)           # Dk = 48: the reference takes its ops path (:271-273)
+    with pytest.raises(DFlashUnsupported):
+        K.tape_replay_kernel(dev(d["v"][..., :16]), dev(d["k"]), dev(d["g"]), dev(d["state"]))
+    d = O.make_gdn_inputs(1, 1, 4, 3, 4, 64, 16)           # Hv % Hk != 0
+    with pytest.raises(DFlashError):
+        K.gated_delta_kernel_with_tape(*(dev(d[n]) for n in ("q", "k", "v", "g", "beta")), dev(d["state"]))
+    with pytest.raises(DFlashError):                        # CPU tensors: there is no CPU path
+        K.tape_replay_kernel(torch.zeros(1, 1, 4, 16), torch.zeros(1, 1, 2, 64), torch.zeros(1, 1, 4),
+                             torch.zeros(1, 4, 16, 64))

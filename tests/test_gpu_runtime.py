@@ -1,0 +1,218 @@
+"""GPU parity for the integer side of the verify step and for the rollback caches:
+acceptance length, commit bookkeeping, conv-window rebuild, KV append, and a full
+arm -> forward -> record -> rollback cycle against the oracle's state machine.
+Integer results are bit-exact; copied bytes are bit-exact; the replayed state is
+held to rtol 1e-4."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import dflash_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+STATE_TOL = dict(rtol=1e-4, atol=1e-6)
+
+
+def dev(a, dt=torch.float32):
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda", dt)
+
+
+def host(t):
+    return t.detach().float().cpu().numpy()
+
+
+def test_match_acceptance_length_bit_exact(gpu_lib):
+    from swiftlm_amd import DFlashRuntime as R
+
+    # the reference's documented example (DFlashRuntime.swift:130-132)
+    got = R.match_acceptance_length(torch.tensor([1, 2, 3], device="cuda"), torch.tensor([1, 2, 5], device="cuda"))
+    assert got.dtype == torch.int32 and int(got) == 2
+    assert int(R.match_acceptance_length(torch.empty(0, dtype=torch.int64, device="cuda"),
+                                         torch.empty(0, dtype=torch.int64, device="cuda"))) == 0
+    rng = np.random.default_rng(0)
+    for n in [1, 2, 15, 16, 63, 64, 65, 200]:
+        for _ in range(6):
+            a = rng.integers(0, 3, n)
+            b = a.copy()
+            if rng.random() < 0.8:
+                b[rng.integers(0, n):] = rng.integers(0, 3)
+            got = int(R.match_acceptance_length(torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()))
+            assert got == O.match_acceptance_length(a, b)
+    # token ids above 2^31 compare as 32-bit patterns
+    big = torch.tensor([4000000000, 7], device="cuda")
+    assert int(R.match_acceptance_length(big, big.clone())) == 2
+
+
+def test_accept_commit_bit_exact(gpu_lib):
+    from swiftlm_amd import DFlashRuntime as R
+
+    rng = np.random.default_rng(1)
+    for _ in range(60):
+        V = int(rng.integers(1, 17))
+        staged = int(rng.integers(0, 50000))
+        drafted = rng.integers(0, 3, V - 1)
+        posterior = rng.integers(0, 3, V)
+        if V > 1 and rng.random() < 0.5:
+            posterior[: V - 1] = drafted                      # fully accepted
+        start = int(rng.integers(0, 100000))
+        verify_ids = torch.tensor([staged] + list(drafted), device="cuda")
+        r = R.accept_commit(verify_ids, torch.from_numpy(posterior).cuda(), start)
+        w = O.accept_commit(staged, drafted, posterior, start)
+        assert (r.acceptance_len, r.commit_count, r.staged_first_next, r.start) == (
+            w["acceptance_len"], w["commit_count"], w["staged_next"], w["start"])
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
+def test_rebuild_conv_state_bit_exact(gpu_lib, dt):
+    import ctypes as C
+
+    from swiftlm_amd import _lib
+
+    B, keep, T, Cc = 2, 3, 16, 8192                           # Qwen3-Next conv width 2*Hk*Dk + Hv*Dv
+    rng = np.random.default_rng(2)
+    snap = dev(rng.standard_normal((B, keep, Cc)).astype(np.float32), dt)
+    qkv = dev(rng.standard_normal((B, T, Cc)).astype(np.float32), dt)
+    lib = _lib.load()
+    for steps in [1, 2, 3, 4, 9, 16]:
+        out = torch.full((B, keep, Cc), 9.0, dtype=dt, device="cuda")
+        rc = lib.dflash_rebuild_conv_state(None, C.c_void_p(snap.data_ptr()), C.c_void_p(qkv.data_ptr()),
+                                           C.c_void_p(out.data_ptr()), B, keep, T, Cc, snap.element_size(), steps, None)
+        assert rc == 0, _lib.last_error()
+        want = O.rebuild_conv_state(host(snap), host(qkv), steps, keep)
+        assert np.array_equal(host(out), want), steps
+    # missing snapshot counts as zeros; step count read on the device
+    sd = torch.tensor([2], dtype=torch.int32, device="cuda")
+    out = torch.full((B, keep, Cc), 9.0, dtype=dt, device="cuda")
+    rc = lib.dflash_rebuild_conv_state(None, None, C.c_void_p(qkv.data_ptr()), C.c_void_p(out.data_ptr()), B, keep, T,
+                                       Cc, snap.element_size(), 0, C.c_void_p(sd.data_ptr()))
+    assert rc == 0
+    assert np.array_equal(host(out), O.rebuild_conv_state(None, host(qkv), 2, keep))
+
+
+def test_kv_append_bit_exact(gpu_lib):
+    import ctypes as C
+
+    from swiftlm_amd import _lib
+
+    B, Hk, M, D, cap = 2, 2, 16, 256, 300
+    g = torch.Generator(device="cuda").manual_seed(3)
+    kc = torch.randn(B, Hk, cap, D, generator=g, device="cuda").bfloat16()
+    vc = torch.randn(B, Hk, cap, D, generator=g, device="cuda").bfloat16()
+    kn = torch.randn(B, Hk, M, D, generator=g, device="cuda").bfloat16()
+    vn = torch.randn(B, Hk, M, D, generator=g, device="cuda").bfloat16()
+    k0, v0 = kc.clone(), vc.clone()
+    lib = _lib.load()
+    p = lambda t: C.c_void_p(t.data_ptr())
+    assert lib.dflash_kv_append(None, p(kc), p(vc), p(kn), p(vn), B, Hk, M, D, 2, Hk * cap * D, cap * D, 100, None,
+                                cap) == 0
+    k0[:, :, 100:116] = kn
+    v0[:, :, 100:116] = vn
+    assert torch.equal(kc, k0) and torch.equal(vc, v0)
+    # offset on the device
+    od = torch.tensor([250], dtype=torch.int32, device="cuda")
+    assert lib.dflash_kv_append(None, p(kc), p(vc), p(kn), p(vn), B, Hk, M, D, 2, Hk * cap * D, cap * D, 0, p(od),
+                                cap) == 0
+    k0[:, :, 250:266] = kn
+    assert torch.equal(kc, k0)
+    # rows outside the capacity are refused on the host
+    assert lib.dflash_kv_append(None, p(kc), p(vc), p(kn), p(vn), B, Hk, M, D, 2, Hk * cap * D, cap * D, 290, None,
+                                cap) == _lib.INVALID
+
+
+def _forward_into_cache(cache, d, qkv, K):
+    q, k, v, g, beta = (dev(d[n], torch.bfloat16) for n in ("q", "k", "v", "g", "beta"))
+    y, s_new, tape = K.gated_delta_kernel_with_tape(q, k, v, g, beta, cache[1])
+    cache[1] = s_new                                           # post-verify state: a new buffer
+    cache[0] = qkv[:, -3:].contiguous()                        # post-verify conv window
+    cache.record_tape(tape, k, g, qkv)
+    return tape
+
+
+@pytest.mark.parametrize("n_accepted", [0, 3, 14])
+def test_recurrent_rollback_cache_cycle(gpu_lib, n_accepted):
+    from swiftlm_amd import DFlashKernels as K, RecurrentRollbackCache
+
+    B, T, Hk, Hv, Dk, Dv, Cc = 1, 16, 16, 32, 128, 128, 8192
+    d = O.make_gdn_inputs(50, B, T, Hk, Hv, Dk, Dv, in_dtype="bf16")
+    rng = np.random.default_rng(5)
+    conv0 = O.round_to_bf16(rng.standard_normal((B, 3, Cc)).astype(np.float32))
+    qkv = O.round_to_bf16(rng.standard_normal((B, T, Cc)).astype(np.float32))
+
+    cache = RecurrentRollbackCache()
+    cache[0] = dev(conv0, torch.bfloat16)
+    cache[1] = dev(d["state"])
+    cache.arm_rollback(prefix_len=100)
+    assert cache.is_armed
+    tape = _forward_into_cache(cache, d, dev(qkv, torch.bfloat16), K)
+    cache.rollback(n_accepted)
+    torch.cuda.synchronize()
+    assert not cache.is_armed
+
+    oc = O.RecurrentRollbackCacheOracle()
+    oc.slots = [conv0, d["state"]]
+    oc.arm_rollback(100)
+    oc.slots = [qkv[:, -3:], None]
+    oc.record_tape(host(tape), d["k"], d["g"], qkv)
+    oc.slots[1] = d["state"]                                   # any non-nil state; rollback restores the snapshot first
+    oc.rollback(n_accepted, dtype=np.float64)
+    np.testing.assert_allclose(host(cache[1]), oc.slots[1], **STATE_TOL)
+    assert np.array_equal(host(cache[0]), oc.slots[0])         # conv window: bit-exact copy
+
+
+def test_restore_target_cache_hybrid_stack(gpu_lib):
+    """A 4-layer hybrid stack (3 GDN + 1 attention) through HybridGDNEngine: partial
+    acceptance replays all tape caches in one launch; full acceptance replays nothing."""
+    from swiftlm_amd import (DFlashKernels as K, HybridGDNEngine, KVCacheSimple, MambaCache,
+                             RecurrentRollbackCache)
+
+    B, T, Hk, Hv, Dk, Dv, Cc = 1, 16, 16, 32, 128, 128, 8192
+    rng = np.random.default_rng(6)
+    engine = HybridGDNEngine()
+    for acceptance_len in (4, 15):
+        caches, ds, qkvs, tapes, conv0s = [], [], [], [], []
+        for layer in range(3):
+            d = O.make_gdn_inputs(60 + layer, B, T, Hk, Hv, Dk, Dv, in_dtype="bf16")
+            c = RecurrentRollbackCache()
+            conv0 = O.round_to_bf16(rng.standard_normal((B, 3, Cc)).astype(np.float32))
+            c[0] = dev(conv0, torch.bfloat16)
+            c[1] = dev(d["state"])
+            caches.append(c); ds.append(d); conv0s.append(conv0)
+        kv = KVCacheSimple(); kv.offset = 1000 + T
+        plain = MambaCache(); plain.offset = 0
+        stack = caches + [kv, plain]
+        engine.arm_rollback(stack, prefix_len=1000)
+        post_states = []
+        for c, d in zip(caches, ds):
+            qkv = O.round_to_bf16(rng.standard_normal((B, T, Cc)).astype(np.float32))
+            tapes.append(_forward_into_cache(c, d, dev(qkv, torch.bfloat16), K)); qkvs.append(qkv)
+            post_states.append(c[1].clone())
+        target_len = 1000 + 1 + acceptance_len
+        ns = engine.rollback(stack, target_len=target_len, acceptance_length=acceptance_len, drafted_tokens=T - 1)
+        torch.cuda.synchronize()
+        assert ns >= 0
+        assert kv.offset == target_len and plain.offset == target_len
+        for c, d, qkv, tape, conv0, post in zip(caches, ds, qkvs, tapes, conv0s, post_states):
+            assert not c.is_armed
+            if acceptance_len == T - 1:                        # fully accepted: keep the forward's state
+                assert torch.equal(c[1], post)
+                assert np.array_equal(host(c[0]), qkv[:, -3:])
+            else:
+                steps = acceptance_len + 1
+                want = O.tape_replay_ops(host(tape)[:, :steps], d["k"][:, :steps], d["g"][:, :steps], d["state"],
+                                         dtype=np.float64)
+                np.testing.assert_allclose(host(c[1]), want, **STATE_TOL)
+                assert np.array_equal(host(c[0]), O.rebuild_conv_state(conv0, qkv, steps, 3))
+
+
+def test_snapshot_cache_restores_pre_verify_state(gpu_lib):
+    from swiftlm_amd import MambaSnapshotCache
+
+    c = MambaSnapshotCache()
+    conv, state = torch.ones(1, 3, 64, device="cuda"), torch.ones(1, 4, 8, 64, device="cuda")
+    c[0], c[1] = conv, state
+    c.arm_rollback(0)
+    c[0], c[1] = conv * 2, state * 2
+    c.rollback(5)
+    assert c[0] is conv and c[1] is state and not c.is_armed

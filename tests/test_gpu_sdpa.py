@@ -1,0 +1,158 @@
+"""GPU parity: block-causal batched GQA SDPA (HIP, through the C ABI) against the
+CPU oracle, and at the long-context sizes against size-independent properties and
+a float32 torch restatement of the same op.
+
+Bar (BASELINE north_star): bf16/f16 outputs within 2e-2 abs/rel; the float32
+logsumexp is held to 2e-3 (its inputs are bf16 products accumulated in fp32)."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle
+from oracle import dflash_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+OUT_TOL = dict(rtol=2e-2, atol=2e-2)
+LSE_TOL = dict(rtol=2e-3, atol=2e-3)
+
+
+def host(t):
+    return t.detach().float().cpu().numpy()
+
+
+def torch_reference(q, k, v, scale, kv_len=None):
+    """float32 restatement on the GPU for sizes the CPU oracle would take minutes on."""
+    B, Hq, M, D = q.shape
+    Hk, N = k.shape[1], k.shape[2]
+    outs, lses = [], []
+    for b in range(B):
+        n = N if kv_len is None else int(kv_len[b])
+        kk = k[b, :, :n].float().repeat_interleave(Hq // Hk, dim=0)
+        vv = v[b, :, :n].float().repeat_interleave(Hq // Hk, dim=0)
+        s = torch.einsum("hmd,hnd->hmn", q[b].float() * scale, kk)
+        vis = torch.arange(n, device=q.device)[None, :] <= (n - M + torch.arange(M, device=q.device))[:, None]
+        s = s.masked_fill(~vis, float("-inf"))
+        lses.append(torch.logsumexp(s, dim=-1))
+        outs.append(torch.einsum("hmn,hnd->hmd", torch.softmax(s, dim=-1), vv))
+    return torch.stack(outs), torch.stack(lses)
+
+
+def gpu_inputs(seed, B, Hq, Hk, L, D, dtype=torch.bfloat16):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    q = torch.randn(B, Hq, 16, D, generator=g, device="cuda").to(dtype)
+    k = torch.randn(B, Hk, L + 16, D, generator=g, device="cuda").to(dtype)
+    v = torch.randn(B, Hk, L + 16, D, generator=g, device="cuda").to(dtype)
+    return q, k, v
+
+
+# (B, Hq, Hk, L, D)
+SMALL = [
+    (1, 16, 2, 0, 256),       # only the block itself: plain causal attention
+    (1, 16, 2, 5, 256),
+    (1, 16, 2, 100, 256),
+    (2, 4, 2, 333, 128),      # group of 2
+    (1, 32, 8, 512, 128),     # the reference bench's shape (DFlashKernelBench/main.swift:201-204)
+    (1, 3, 3, 70, 128),       # no grouping, odd head count
+    (1, 24, 2, 200, 128),     # group of 12: two workgroups per KV head
+    (1, 16, 2, 1000, 256),
+]
+
+
+@pytest.mark.parametrize("cfg", SMALL, ids=[f"B{c[0]}_Hq{c[1]}_Hk{c[2]}_L{c[3]}_D{c[4]}" for c in SMALL])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_sdpa_matches_oracle_small(gpu_lib, cfg, dtype):
+    from swiftlm_amd import DFlashKernels as K
+
+    B, Hq, Hk, L, D = cfg
+    q, k, v = gpu_inputs(B * 1000 + L, B, Hq, Hk, L, D, dtype)
+    scale = 1.0 / math.sqrt(D)
+    out, lse = K.batched_sdpa_2pass(q, k, v, scale, return_lse=True)
+    torch.cuda.synchronize()
+    ow, lw = O.sdpa_block_causal(host(q), host(k), host(v), scale)
+    assert out.dtype == dtype and out.shape == q.shape and lse.shape == (B, Hq, 16)
+    np.testing.assert_allclose(host(out), ow, **OUT_TOL)
+    np.testing.assert_allclose(host(lse), lw, **LSE_TOL)
+
+
+def test_sdpa_config2_against_c_oracle(gpu_lib):
+    """BASELINE config 2: Hq=16, Hkv=2, D=256, L=4096, scale 1/16."""
+    from swiftlm_amd import DFlashKernels as K
+
+    q, k, v = gpu_inputs(2, 1, 16, 2, 4096, 256)
+    out, lse = K.batched_sdpa_2pass(q, k, v, 1.0 / 16, return_lse=True)
+    ow, lw = c_oracle.sdpa_block_causal(host(q), host(k), host(v), 1.0 / 16)
+    np.testing.assert_allclose(host(out), ow, **OUT_TOL)
+    np.testing.assert_allclose(host(lse), lw, **LSE_TOL)
+    # without LSE the result is the same array
+    assert torch.equal(K.batched_sdpa_2pass(q, k, v, 1.0 / 16), out)
+    # inputs untouched, K/V taken as a view into a larger cache
+    cache_k = torch.zeros(1, 2, 8192, 256, dtype=torch.bfloat16, device="cuda")
+    cache_v = torch.zeros_like(cache_k)
+    cache_k[:, :, :4112] = k
+    cache_v[:, :, :4112] = v
+    out2 = K.batched_sdpa_2pass(q, cache_k[:, :, :4112], cache_v[:, :, :4112], 1.0 / 16)
+    assert torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("L", [32768, 40960, 102400])
+def test_sdpa_long_context_properties(gpu_lib, L):
+    """BASELINE config 3 sizes.  Properties that do not need a CPU pass: constant V gives
+    constant O; the result matches a float32 restatement; appending hidden (future) keys
+    changes nothing for the rows that cannot see them."""
+    from swiftlm_amd import DFlashKernels as K
+
+    q, k, v = gpu_inputs(L, 1, 16, 2, L, 256)
+    out, lse = K.batched_sdpa_2pass(q, k, v, 1.0 / 16, return_lse=True)
+    ow, lw = torch_reference(q, k, v, 1.0 / 16)
+    np.testing.assert_allclose(host(out), host(ow), **OUT_TOL)
+    np.testing.assert_allclose(host(lse), host(lw), **LSE_TOL)
+    const = K.batched_sdpa_2pass(q, k, torch.full_like(v, 0.75), 1.0 / 16)
+    np.testing.assert_allclose(host(const), 0.75, rtol=1e-2)
+    # row 0 sees keys 0..L only: changing the last 15 keys must not move it
+    k2, v2 = k.clone(), v.clone()
+    k2[:, :, L + 1:] = 3.0
+    v2[:, :, L + 1:] = -5.0
+    out2 = K.batched_sdpa_2pass(q, k2, v2, 1.0 / 16)
+    assert torch.equal(out2[:, :, 0], out[:, :, 0])
+
+
+def test_sdpa_ragged_batch(gpu_lib):
+    """BASELINE config 3's ragged batch: 4 sequences with L ~ U[8K, 64K], one launch,
+    per-sequence key counts on the device."""
+    from swiftlm_amd import DFlashKernels as K
+
+    rng = np.random.default_rng(0)
+    Ls = rng.integers(8192, 65536, 4)
+    Nmax = int(Ls.max()) + 16
+    q, k, v = gpu_inputs(77, 4, 16, 2, Nmax - 16, 256)
+    kv_len = torch.tensor([int(l) + 16 for l in Ls], dtype=torch.int32, device="cuda")
+    out, lse = K.batched_sdpa_2pass(q, k, v, 1.0 / 16, return_lse=True, kv_len=kv_len)
+    ow, lw = torch_reference(q, k, v, 1.0 / 16, kv_len=kv_len.tolist())
+    np.testing.assert_allclose(host(out), host(ow), **OUT_TOL)
+    np.testing.assert_allclose(host(lse), host(lw), **LSE_TOL)
+    # each sequence alone gives the same rows
+    for b in (0, 3):
+        n = int(kv_len[b])
+        single = K.batched_sdpa_2pass(q[b:b + 1], k[b:b + 1, :, :n].contiguous(), v[b:b + 1, :, :n].contiguous(),
+                                      1.0 / 16)
+        np.testing.assert_allclose(host(single), host(out[b:b + 1]), rtol=1e-2, atol=1e-2)
+
+
+def test_sdpa_unsupported_shapes_return_none(gpu_lib):
+    """The reference's guards (DFlashKernels.swift:744-758): nil instead of an error."""
+    from swiftlm_amd import DFlashKernels as K, DFlashUnsupported
+
+    q, k, v = gpu_inputs(1, 1, 4, 2, 64, 128)
+    assert K.batched_sdpa_2pass(q[:, :, :8], k, v, 0.1) is None                  # qLen != 16
+    assert K.batched_sdpa_2pass(q.float(), k.float(), v.float(), 0.1) is None    # float32
+    q64, k64, v64 = gpu_inputs(1, 1, 4, 2, 64, 64)
+    assert K.batched_sdpa_2pass(q64, k64, v64, 0.1) is None                      # D = 64
+    q3, _, _ = gpu_inputs(1, 1, 3, 2, 64, 128)
+    assert K.batched_sdpa_2pass(q3, k, v, 0.1) is None                           # Hq % Hk != 0
+    assert K.batched_sdpa_2pass(q[0], k[0], v[0], 0.1) is None                   # ndim != 4
+    with pytest.raises(DFlashUnsupported):
+        K.sdpa_fallback(q64, k64, v64, 0.1)
