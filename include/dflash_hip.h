@@ -186,12 +186,30 @@ int dflash_rebuild_conv_state(void* stream, const void* snapshot_conv, const voi
  * KV append for an attention layer at verify (the KVCacheSimple.update the
  * reference delegates to mlx-swift-lm, trimmed by DFlashRuntime.swift:212-218):
  * copies k_new/v_new [B, Hk, M, D] to rows [offset, offset+M) of a cache laid out
- * like k/v above.  offset comes from *offset_dev when not NULL.
+ * like k/v above.  offset comes from *offset_dev when not NULL.  new_len_dev, when
+ * not NULL, receives offset + M (the cache's length after the append, which is
+ * the N of the attention call that follows).  An append that would pass the
+ * capacity writes nothing.
  * ---------------------------------------------------------------------- */
 int dflash_kv_append(void* stream, void* k_cache, void* v_cache, const void* k_new, const void* v_new,
                      int B, int Hk, int M, int D, int elem_bytes,
                      int64_t kv_batch_stride, int64_t kv_head_stride,
-                     int offset, const int32_t* offset_dev, int capacity);
+                     int offset, const int32_t* offset_dev, int capacity, int32_t* new_len_dev);
+
+/* ------------------------------------------------------------------------
+ * Measurement hook (no counterpart in the reference, whose bench times whole
+ * calls from the host: Sources/DFlashKernelBench/main.swift:33-57).  Arms the
+ * calling thread so that the NEXT launch of the named kernel is bracketed by
+ * hipEventRecord(start_event) / hipEventRecord(stop_event) on the launch stream;
+ * the arming is consumed by that launch.  Events are hipEvent_t passed as void*,
+ * created and read by the caller.
+ * ---------------------------------------------------------------------- */
+#define DFLASH_KERNEL_SDPA_PARTIAL 0
+#define DFLASH_KERNEL_SDPA_COMBINE 1
+#define DFLASH_KERNEL_GDN_FORWARD 2
+#define DFLASH_KERNEL_TAPE_REPLAY 3
+#define DFLASH_KERNEL_COUNT 4
+int dflash_profile_next_launch(int kernel_id, void* start_event, void* stop_event);
 
 #ifdef __cplusplus
 }

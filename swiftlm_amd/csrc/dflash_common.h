@@ -45,6 +45,17 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 int ensure_init();           // per-device one-time setup; 0 or negative hip error
 int num_compute_units();     // of the current device (cached)
 
+// Brackets one kernel launch with the caller's events when the thread was armed by
+// dflash_profile_next_launch(); otherwise does nothing.
+struct LaunchBracket {
+    hipStream_t stream;
+    hipEvent_t stop;
+    LaunchBracket(int kernel_id, hipStream_t st);
+    ~LaunchBracket() { if (stop) (void)hipEventRecord(stop, stream); }
+    LaunchBracket(const LaunchBracket&) = delete;
+    LaunchBracket& operator=(const LaunchBracket&) = delete;
+};
+
 inline int dtype_size(int dt) {
     switch (dt) {
         case DFLASH_F32: return 4;

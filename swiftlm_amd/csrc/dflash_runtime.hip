@@ -47,6 +47,19 @@ int num_compute_units() {
     return g_cus[dev];
 }
 
+// ---- measurement hook --------------------------------------------------------
+
+struct ArmedBracket { hipEvent_t start = nullptr, stop = nullptr; };
+static thread_local ArmedBracket g_bracket[DFLASH_KERNEL_COUNT];
+
+LaunchBracket::LaunchBracket(int kernel_id, hipStream_t st) : stream(st), stop(nullptr) {
+    ArmedBracket& a = g_bracket[kernel_id];
+    if (!a.start) return;
+    (void)hipEventRecord(a.start, st);
+    stop = a.stop;
+    a.start = a.stop = nullptr;
+}
+
 // ---- acceptance ------------------------------------------------------------
 
 // One wave.  Leading-match count = index of the first mismatch (n if none);
@@ -107,9 +120,10 @@ __global__ __launch_bounds__(256) void rebuild_conv_kernel(const uint4* snap, co
 __global__ __launch_bounds__(256) void kv_append_kernel(uint4* k_cache, uint4* v_cache, const uint4* k_new,
                                                         const uint4* v_new, int Hk, int M, int D16, long batch_stride16,
                                                         long head_stride16, int offset, const int32_t* offset_dev,
-                                                        int capacity) {
+                                                        int capacity, int32_t* new_len_dev) {
     int off = offset_dev ? *offset_dev : offset;
     if (off < 0 || off + M > capacity) return;   // never write outside the cache
+    if (new_len_dev && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *new_len_dev = off + M;
     const int bh = blockIdx.y;
     const int b = bh / Hk, hk = bh % Hk;
     const int per = M * D16;
@@ -128,6 +142,14 @@ using namespace dflash;
 extern "C" int dflash_version(void) { return 100; }
 extern "C" const char* dflash_last_error(void) { return g_err; }
 extern "C" int dflash_init(void) { return ensure_init(); }
+
+extern "C" int dflash_profile_next_launch(int kernel_id, void* start_event, void* stop_event) {
+    DFLASH_REQUIRE(kernel_id >= 0 && kernel_id < DFLASH_KERNEL_COUNT, "profile_next_launch: bad kernel id %d", kernel_id);
+    DFLASH_REQUIRE((start_event == nullptr) == (stop_event == nullptr), "profile_next_launch: pass both events or neither");
+    g_bracket[kernel_id].start = (hipEvent_t)start_event;
+    g_bracket[kernel_id].stop = (hipEvent_t)stop_event;
+    return DFLASH_OK;
+}
 
 extern "C" int dflash_match_acceptance_length(void* stream, const uint32_t* drafted, const uint32_t* posterior, int n,
                                               int32_t* out) {
@@ -171,7 +193,7 @@ extern "C" int dflash_rebuild_conv_state(void* stream, const void* snapshot_conv
 
 extern "C" int dflash_kv_append(void* stream, void* k_cache, void* v_cache, const void* k_new, const void* v_new, int B,
                                 int Hk, int M, int D, int elem_bytes, int64_t kv_batch_stride, int64_t kv_head_stride,
-                                int offset, const int32_t* offset_dev, int capacity) {
+                                int offset, const int32_t* offset_dev, int capacity, int32_t* new_len_dev) {
     int rc = ensure_init();
     if (rc) return rc;
     DFLASH_REQUIRE(k_cache && v_cache && k_new && v_new, "kv_append: null pointer");
@@ -188,7 +210,7 @@ extern "C" int dflash_kv_append(void* stream, void* k_cache, void* v_cache, cons
     dim3 grid((M * D16 + 255) / 256, B * Hk);
     hipLaunchKernelGGL(kv_append_kernel, grid, dim3(256), 0, (hipStream_t)stream, (uint4*)k_cache, (uint4*)v_cache,
                        (const uint4*)k_new, (const uint4*)v_new, Hk, M, D16, (long)(kv_batch_stride * elem_bytes / 16),
-                       (long)(kv_head_stride * elem_bytes / 16), offset, offset_dev, capacity);
+                       (long)(kv_head_stride * elem_bytes / 16), offset, offset_dev, capacity, new_len_dev);
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
 }

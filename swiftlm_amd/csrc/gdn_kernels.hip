@@ -156,6 +156,7 @@ static int launch_replay_nr(hipStream_t st, const ReplayBatch& P, const ReplayAr
     // Fewer, fatter workgroups once the grid already covers the chip several times over.
     const long wg1 = (long)((A.Dv + RPP - 1) / RPP) * B * A.Hv * n_layers;
     const int cus = num_compute_units();
+    LaunchBracket br(DFLASH_KERNEL_TAPE_REPLAY, st);
     if (wg1 >= 16L * cus && A.Dv >= RPP * 4) {
         dim3 grid((A.Dv + RPP * 4 - 1) / (RPP * 4), B * A.Hv, n_layers);
         hipLaunchKernelGGL((tape_replay_kernel<StateT, VEC_G, DK, 4>), grid, dim3(kThreads), 0, st, P, A);
@@ -374,6 +375,7 @@ static int launch_gdn_state(hipStream_t st, const GdnArgs& A, int B, int g_ndim,
 #define DFLASH_GDN_CASE(DKV, LPRV)                                                                     \
     case DKV: {                                                                                        \
         dim3 grid((A.Dv + (kThreads / LPRV) - 1) / (kThreads / LPRV), B * A.Hv);                       \
+        LaunchBracket br(DFLASH_KERNEL_GDN_FORWARD, st);                                               \
         if (vec) hipLaunchKernelGGL((gated_delta_tape_kernel<StateT, true, DKV, LPRV>), grid, dim3(kThreads), 0, st, A); \
         else hipLaunchKernelGGL((gated_delta_tape_kernel<StateT, false, DKV, LPRV>), grid, dim3(kThreads), 0, st, A);    \
         DFLASH_HIP_TRY(hipGetLastError());                                                             \

@@ -39,10 +39,12 @@ typedef __attribute__((ext_vector_type(8))) float f32x8_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;   // one 16-byte global/LDS access
 
 constexpr int kSdpaThreads = 256;
-constexpr int kBN = 64;             // keys per tile
+constexpr int kBN = 32;             // keys per tile
+constexpr int kStages = 4;          // LDS tile buffers in flight
 constexpr int kM = 16;              // block rows per head
 constexpr int kHeadsPerWG = 8;      // query heads sharing one K/V pass
 constexpr int kMaxSplits = 512;
+constexpr float kRescaleLog2 = 8.f;   // lazy-rescale threshold of the online softmax, log2 units
 
 struct Bf16Tag {
     typedef bf16x8_t vec8;
@@ -51,6 +53,7 @@ struct Bf16Tag {
     }
     static __device__ __forceinline__ vec8 pack(f32x8_t x) { return __builtin_convertvector(x, vec8); }
     static __device__ __forceinline__ uint16_t cvt(float x) { return f32_to_bf16_bits(x); }
+    static __device__ __forceinline__ float to_f32(uint16_t x) { return __uint_as_float(((uint32_t)x) << 16); }
 };
 struct F16Tag {
     typedef f16x8_t vec8;
@@ -62,13 +65,14 @@ struct F16Tag {
         _Float16 hf = (_Float16)x;
         return *reinterpret_cast<uint16_t*>(&hf);
     }
+    static __device__ __forceinline__ float to_f32(uint16_t x) { return (float)__builtin_bit_cast(_Float16, x); }
 };
 
 struct SdpaArgs {
     const uint16_t* q;
     const uint16_t* k;
     const uint16_t* v;
-    float* part_o;   // [B*Hq*16, S, D]
+    uint16_t* part_o;   // [B*Hq*16, S, D]  unnormalised partial O in the input type (DFlashKernels.swift:647)
     float* part_m;   // [B*Hq*16, S]   running max, log2 units
     float* part_l;   // [B*Hq*16, S]   sum of exp2
     const int32_t* kv_len_dev;
@@ -77,34 +81,71 @@ struct SdpaArgs {
     int Hq, Hk, G, N, S, groups_per_kv;
 };
 
+// LDS plan of the partial kernel.  A stage holds one tile of kBN keys: the K rows
+// followed by the V rows, both row-major [key][D] exactly as in HBM but with the
+// 16-byte pieces of each row permuted (XOR swizzle) so that the MFMA operand reads
+// below hit every bank once.  kStages stages are in flight.
 template <int D> struct SdpaLds {
-    static constexpr int KS = D + 8;           // K row stride, elements
-    static constexpr int VS = kBN + 8;         // V^T row stride, elements
-    static constexpr int K_BYTES = kBN * KS * 2;
-    static constexpr int V_BYTES = D * VS * 2;
-    static constexpr int STAGE = K_BYTES + V_BYTES;
-    static constexpr int OS = D + 4;           // epilogue O row stride, floats
+    static constexpr int ROWB = D * 2;               // bytes per K or V row
+    static constexpr int CPR = D / 8;                // 16-byte pieces per row
+    static constexpr int RPI = 64 / CPR;             // rows covered by one wave-wide 1 KB load
+    static constexpr int K_BYTES = kBN * ROWB;
+    static constexpr int STAGE = 2 * K_BYTES;
+    static constexpr int LPW = (kBN / RPI) / 4;      // load instructions per wave per tile and operand
+    static constexpr int OS = D + 4;                 // epilogue O row stride, floats
     static constexpr int EPI = 4 * 32 * OS * 4;
-    static constexpr int BYTES = 2 * STAGE > EPI ? 2 * STAGE : EPI;
+    static constexpr int BYTES = kStages * STAGE > EPI ? kStages * STAGE : EPI;
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(8))) short s16x8_t;
+
+// 64 lanes x 16 B from HBM straight into LDS at lds_base + 16 * lane (lds_base is wave-uniform and
+// travels in M0).  Issued as inline assembly on purpose: the compiler then does not track these
+// loads, so it cannot force a full vmcnt(0) drain ahead of every LDS read or barrier; completion
+// is tracked by hand with wait_vmcnt<> below, which is what keeps several tiles in flight.
+__device__ __forceinline__ void async_load_16B(const unsigned char* gbase, uint32_t goff, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(goff), "s"(gbase), "s"(lds_base)
+                 : "memory", "m0");
+}
+
+// s_waitcnt vmcnt(n) only (expcnt and lgkmcnt left alone), GFX9 encoding.
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt(((N >> 4) << 14) | (0xF << 8) | (0x7 << 4) | (N & 0xF));
+}
+
 // Grid: x = split, y = kv head * groups_per_kv + head group, z = batch.
+//
+// Data movement: K/V rows go HBM -> LDS directly (global_load_lds_dwordx4, no VGPR
+// staging), kStages-1 tiles ahead of the tile being multiplied.  A wave-wide load
+// deposits 64 x 16 B contiguously in LDS in lane order, so the swizzle is applied on
+// the way in: lane l, which fills piece l % CPR of its row, fetches piece
+// (l % CPR) ^ f(row) from HBM.  K uses f = row % 16 (conflict-free ds_read_b128 of
+// one piece per key row across 16 lanes); V uses f = 4 * (row % 4) (conflict-free
+// ds_read_b64_tr_b16 of 4 key rows x 32 B per 16-lane group).
+// V^T operands come from the transposing LDS read: in each 16-lane group, lane
+// 4*j + q supplies the address of 4 channels of key row j; lane i receives channel
+// (i % 4) of the address given by lane 4*r + i/4 as its r-th element, i.e. four
+// consecutive keys of channel d0 + i when lane 4*j + q points at V[k0 + j][d0 + 4q].
 template <typename Tag, int D>
 __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs A) {
     typedef typename Tag::vec8 vec8;
     typedef SdpaLds<D> L;
     constexpr int KSTEPS = D / 16;     // MFMA k-steps over the head dimension
     constexpr int DB = D / 32;         // 32-wide output blocks over the head dimension
-    constexpr int KCH = (kBN * D / 8) / kSdpaThreads;   // 16-byte K chunks per thread per tile
-    constexpr int VBLK = (kBN / 8) * (D / 8);           // 8x8 V blocks per tile
-    static_assert(VBLK <= kSdpaThreads, "one V block per thread");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    // LDS byte address of smem (what M0 and the ds_* instructions use)
+    const uint32_t smem_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane & 31, h = lane >> 5;
     const int split = blockIdx.x;
     const int hk = blockIdx.y / A.groups_per_kv;
@@ -134,8 +175,38 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
         return;
     }
 
-    const uint16_t* kbase = A.k + (size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride;
-    const uint16_t* vbase = A.v + (size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride;
+    const unsigned char* kbase = reinterpret_cast<const unsigned char*>(A.k) +
+                                 ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
+    const unsigned char* vbase = reinterpret_cast<const unsigned char*>(A.v) +
+                                 ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
+
+    // ---- asynchronous tile loads ------------------------------------------------
+    // Load instruction j of this wave covers rows (4*j + wave) * RPI .. + RPI - 1 of the tile.
+    const int ld_rsub = lane / L::CPR;           // row within the instruction's row group
+    const int ld_pos = lane % L::CPR;            // 16-byte slot this lane fills
+    auto issue_tile = [&](int t) {
+        const uint32_t stage_lds = smem_lds + ((t - t_begin) % kStages) * L::STAGE;
+        const int key0 = t * kBN;
+#pragma unroll
+        for (int j = 0; j < L::LPW; ++j) {
+            const int rg = (4 * j + wave) * L::RPI;
+            const int row = rg + ld_rsub;
+            int key = key0 + row;
+            key = key < Nb ? key : Nb - 1;
+            const uint32_t goff_k = (uint32_t)key * L::ROWB + (uint32_t)((ld_pos ^ (row & 15)) * 16);
+            const uint32_t goff_v = (uint32_t)key * L::ROWB + (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
+            async_load_16B(kbase, goff_k, stage_lds + rg * L::ROWB);
+            async_load_16B(vbase, goff_v, stage_lds + L::K_BYTES + rg * L::ROWB);
+        }
+    };
+    constexpr int LD_PER_TILE = 2 * L::LPW;      // vmcnt events per tile and wave
+
+    // The first kStages-1 tiles go out before anything else so that Q and the tiles share one
+    // memory round trip.  (Older loads retire first, so the compiler's own vmcnt waits for Q,
+    // which count only its loads, are conservative and stay correct.)
+#pragma unroll
+    for (int i = 0; i < kStages - 1; ++i)
+        if (t_begin + i < t_end) issue_tile(t_begin + i);
 
     // ---- Q as B operands: column c = query row, k-elements 16*s + 8h .. +7 ----
     vec8 qreg[KSTEPS];
@@ -148,6 +219,10 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
             qreg[s] = __builtin_bit_cast(vec8, u);
         }
     }
+    // Q must be complete here, and the compiler must know it: it does not see the asynchronous
+    // tile loads, so a Q wait left to it lands on the first MFMA INSIDE the loop as a full
+    // vmcnt(0) drain per tile, which serialises loading and computing.
+    wait_vmcnt<0>();
 
     f32x16_t oacc[DB];
 #pragma unroll
@@ -156,79 +231,47 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
         for (int v = 0; v < 16; ++v) oacc[i][v] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
 
-    u32x4_t kreg[KCH];
-    u32x4_t vreg[8];
-    // V block owned by this thread: 8 keys (one LDS position group) x 8 channels
-    const int v_kg = tid & 7, v_dc = tid >> 3;
-    const int v_keybase = 32 * (v_kg >> 2) + 16 * ((v_kg >> 1) & 1) + 4 * (v_kg & 1);
-
-    auto load_tile = [&](int t) {
-        const int key0 = t * kBN;
-#pragma unroll
-        for (int j = 0; j < KCH; ++j) {
-            const int id = tid + kSdpaThreads * j;
-            int key = key0 + id / (D / 8);
-            key = key < Nb ? key : Nb - 1;
-            kreg[j] = *reinterpret_cast<const u32x4_t*>(kbase + (size_t)key * D + (id % (D / 8)) * 8);
-        }
-        if (VBLK == kSdpaThreads || tid < VBLK) {
-#pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                int key = key0 + v_keybase + 8 * (r >> 2) + (r & 3);
-                key = key < Nb ? key : Nb - 1;
-                vreg[r] = *reinterpret_cast<const u32x4_t*>(vbase + (size_t)key * D + v_dc * 8);
-            }
-        }
-    };
-    auto store_tile = [&](int buf) {
-        uint16_t* ks = reinterpret_cast<uint16_t*>(smem + buf * L::STAGE);
-        uint16_t* vt = reinterpret_cast<uint16_t*>(smem + buf * L::STAGE + L::K_BYTES);
-#pragma unroll
-        for (int j = 0; j < KCH; ++j) {
-            const int id = tid + kSdpaThreads * j;
-            *reinterpret_cast<u32x4_t*>(ks + (id / (D / 8)) * L::KS + (id % (D / 8)) * 8) = kreg[j];
-        }
-        if (VBLK == kSdpaThreads || tid < VBLK) {
-            // 8x8 transpose of 16-bit elements: row r of vreg is key r, we need channel dd -> 8 keys
-#pragma unroll
-            for (int dd = 0; dd < 8; ++dd) {
-                u32x4_t w;
-#pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    const uint32_t lo = vreg[2 * p][dd >> 1];
-                    const uint32_t hi = vreg[2 * p + 1][dd >> 1];
-                    w[p] = (dd & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
-                }
-                *reinterpret_cast<u32x4_t*>(vt + (v_dc * 8 + dd) * L::VS + v_kg * 8) = w;
-            }
-        }
-    };
-
-    load_tile(t_begin);
-    store_tile(0);
-    __syncthreads();
+    // per-lane pieces of the operand addresses
+    const int k_rd = c * L::ROWB;                        // K: this lane's key row
+    const int k_sw = c & 15;
+    const int tj = (lane & 15) >> 2, tq = lane & 3;      // V: transposing read, lane = 4*tj + tq in its group
+    const int tg = lane >> 4;                            // group: channel half tg & 1, key half tg >> 1
+    const int v_rd = (4 * (tg >> 1) + tj) * L::ROWB + (tq & 1) * 8;
+    const int v_piece = 2 * (tg & 1) + (tq >> 1);        // 16-byte piece within a 32-channel block
+    const int v_sw = 4 * tj;                             // row % 4 == tj for every row this lane reads
 
     for (int t = t_begin; t < t_end; ++t) {
-        const int buf = (t - t_begin) & 1;
-        const bool more = (t + 1) < t_end;
-        if (more) load_tile(t + 1);
+        // tile t has landed once at most (tiles issued after it) * LD_PER_TILE loads are outstanding
+        const int ahead = (t_end - 1 - t) < (kStages - 2) ? (t_end - 1 - t) : (kStages - 2);
+        if (ahead >= 2) wait_vmcnt<2 * LD_PER_TILE>();
+        else if (ahead == 1) wait_vmcnt<LD_PER_TILE>();
+        else wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();   // everyone's share of tile t is in LDS; everyone is done with tile t-1
+        if (t + kStages - 1 < t_end) issue_tile(t + kStages - 1);   // refills the stage tile t-1 used
 
         if (wave_active) {
-            const uint16_t* ks = reinterpret_cast<const uint16_t*>(smem + buf * L::STAGE);
-            const uint16_t* vt = reinterpret_cast<const uint16_t*>(smem + buf * L::STAGE + L::K_BYTES);
+            const unsigned char* ks = smem + ((t - t_begin) % kStages) * L::STAGE;
+            const unsigned char* vs = ks + L::K_BYTES;
 
-            // ---- S^T = K Q^T for the tile's two 32-key blocks ----
-            f32x16_t sacc[2];
+            // ---- S^T = K Q^T for the tile's 32 keys ----
+            f32x16_t sacc;
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
+            for (int v = 0; v < 16; ++v) sacc[v] = 0.f;
+            vec8 ka[KSTEPS];
 #pragma unroll
-                for (int v = 0; v < 16; ++v) sacc[kb][v] = 0.f;
+            for (int s = 0; s < KSTEPS; ++s)
+                ka[s] = *reinterpret_cast<const vec8*>(ks + k_rd + (((2 * s + h) ^ k_sw) * 16));
 #pragma unroll
-                for (int s = 0; s < KSTEPS; ++s) {
-                    const vec8 a = *reinterpret_cast<const vec8*>(ks + (32 * kb + c) * L::KS + 16 * s + 8 * h);
-                    sacc[kb] = Tag::mfma(a, qreg[s], sacc[kb]);
-                }
+            for (int s = 0; s < KSTEPS; ++s) sacc = Tag::mfma(ka[s], qreg[s], sacc);
+            // Issue order for the block above: half of the operand reads up front, then one read per
+            // MFMA, so the LDS latency hides behind the matrix pipe instead of stalling every MFMA.
+            __builtin_amdgcn_sched_group_barrier(0x100, KSTEPS / 2, 0);
+#pragma unroll
+            for (int s = 0; s < KSTEPS / 2; ++s) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             }
+            __builtin_amdgcn_sched_group_barrier(0x008, KSTEPS / 2, 0);
 
             // ---- scale, causal mask, online softmax (log2 domain) ----
             const int key0 = t * kBN;
@@ -236,33 +279,34 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
             const int last_visible = Nb - kM + qi;     // row qi sees keys 0 .. Nb-16+qi
             float mloc = -INFINITY;
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    float x = sacc[kb][v] * A.scale_log2;
-                    if (need_mask) {
-                        const int key = key0 + 32 * kb + 8 * (v >> 2) + 4 * h + (v & 3);
-                        x = key <= last_visible ? x : -INFINITY;
-                    }
-                    sacc[kb][v] = x;
-                    mloc = fmaxf(mloc, x);
+            for (int v = 0; v < 16; ++v) {
+                float x = sacc[v] * A.scale_log2;
+                if (need_mask) {
+                    const int key = key0 + 8 * (v >> 2) + 4 * h + (v & 3);
+                    x = key <= last_visible ? x : -INFINITY;
                 }
+                sacc[v] = x;
+                mloc = fmaxf(mloc, x);
+            }
             mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-            const float m_new = fmaxf(m_run, mloc);
+            // Lazy rescale: the exponent reference m_run only moves when the tile's maximum
+            // exceeds it by more than kRescaleLog2 (P then stays below 2^kRescaleLog2, harmless in
+            // fp32/bf16), so the 128 accumulator registers are rarely touched by the softmax.
+            const bool bump = mloc > m_run + kRescaleLog2;      // also true for the first finite maximum
+            const float m_new = bump ? mloc : m_run;
             const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = fast_exp2(m_run - m_safe);
+            const float alpha = bump ? fast_exp2(m_run - m_safe) : 1.f;
+            const bool rescale = bump && m_run != -INFINITY;    // nothing accumulated yet otherwise
             m_run = m_new;
             float psum = 0.f;
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const float p = fast_exp2(sacc[kb][v] - m_safe);
-                    sacc[kb][v] = p;
-                    psum += p;
-                }
+            for (int v = 0; v < 16; ++v) {
+                const float p = fast_exp2(sacc[v] - m_safe);
+                sacc[v] = p;
+                psum += p;
+            }
             l_run = l_run * alpha + psum;
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+            if (__builtin_amdgcn_ballot_w64(rescale) != 0) {
 #pragma unroll
                 for (int i = 0; i < DB; ++i)
 #pragma unroll
@@ -270,25 +314,28 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
             }
 
             // ---- O^T += V^T P^T ----
+            // MFMA ksub feeds accumulator registers 8*ksub .. 8*ksub+7, i.e. keys
+            // 16*ksub + {4h..4h+3} and 16*ksub + 8 + {4h..4h+3}: two transposing reads.
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int ksub = 0; ksub < 2; ++ksub) {
+                f32x8_t pf;
 #pragma unroll
-                for (int ksub = 0; ksub < 2; ++ksub) {
-                    f32x8_t pf;
+                for (int e = 0; e < 8; ++e) pf[e] = sacc[8 * ksub + e];
+                const vec8 pb = Tag::pack(pf);
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) pf[e] = sacc[kb][8 * ksub + e];
-                    const vec8 pb = Tag::pack(pf);
-#pragma unroll
-                    for (int i = 0; i < DB; ++i) {
-                        const vec8 a = *reinterpret_cast<const vec8*>(vt + (32 * i + c) * L::VS + 32 * kb + 16 * ksub + 8 * h);
-                        oacc[i] = Tag::mfma(a, pb, oacc[i]);
-                    }
+                for (int i = 0; i < DB; ++i) {
+                    const int off = v_rd + ((((4 * i + v_piece)) ^ v_sw) * 16);
+                    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) s16x4_t*)(vs + off + (16 * ksub) * L::ROWB));
+                    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) s16x4_t*)(vs + off + (16 * ksub + 8) * L::ROWB));
+                    const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    oacc[i] = Tag::mfma(__builtin_bit_cast(vec8, both), pb, oacc[i]);
                 }
+            }
         }
-
-        if (more) store_tile(buf ^ 1);
-        __syncthreads();
     }
+    __syncthreads();          // the tile buffers are free for the epilogue
 
     // ---- epilogue: partial statistics and O rows (through LDS for coalesced stores) ----
     const float l_tot = l_run + __shfl_xor(l_run, 32);
@@ -307,20 +354,30 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
             }
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): LDS writes of this wave are visible to it
-        for (int r = 0; r < 32; ++r) {
-            const int head = 2 * wave + (r >> 4);
-            if (head >= hcount) break;
-            const size_t rid = ((size_t)b * A.Hq + hk * A.G + hg0 + head) * kM + (r & 15);
-            float* dst = A.part_o + (rid * A.S + split) * D;
-            for (int d = lane * 4; d < D; d += 256)
-                *reinterpret_cast<float4*>(dst + d) = *reinterpret_cast<const float4*>(os + r * L::OS + d);
+        const int rows = (hcount - 2 * wave) >= 2 ? 32 : 16;        // this wave's valid rows (whole heads)
+        const size_t rid0 = ((size_t)b * A.Hq + hk * A.G + hg0 + 2 * wave) * kM;   // rows are consecutive
+        constexpr int PER_ROW = D / 4;                              // lanes per row, 4 channels each
+        constexpr int RPP = 64 / PER_ROW > 0 ? 64 / PER_ROW : 1;    // rows per pass of the wave
+        const int rsub = lane / PER_ROW, d = (lane % PER_ROW) * 4;
+        for (int r0 = 0; r0 < rows; r0 += 8 * RPP) {
+            float4 o[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) o[u] = *reinterpret_cast<const float4*>(os + (r0 + u * RPP + rsub) * L::OS + d);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int r = r0 + u * RPP + rsub;
+                uint2 pk;
+                pk.x = (uint32_t)Tag::cvt(o[u].x) | ((uint32_t)Tag::cvt(o[u].y) << 16);
+                pk.y = (uint32_t)Tag::cvt(o[u].z) | ((uint32_t)Tag::cvt(o[u].w) << 16);
+                if (r < rows) *reinterpret_cast<uint2*>(A.part_o + ((rid0 + r) * A.S + split) * D + d) = pk;
+            }
         }
     }
 }
 
 // One workgroup per output row (b, hq, i): merges the S partials.
 struct CombineArgs {
-    const float* part_o;
+    const uint16_t* part_o;
     const float* part_m;
     const float* part_l;
     uint16_t* out;
@@ -330,11 +387,12 @@ struct CombineArgs {
 
 template <typename Tag, int D>
 __global__ __launch_bounds__(kSdpaThreads) void sdpa_combine_kernel(CombineArgs A) {
-    constexpr int TPG = D / 4;                     // threads spanning one row as float4
+    constexpr int TPG = D / 8;                     // threads spanning one row, 8 elements (16 B) each
     constexpr int NG = kSdpaThreads / TPG;         // split groups walking the partials in parallel
+    constexpr int UNROLL = 4;
     __shared__ float w_s[kMaxSplits];
     __shared__ float red_s[kSdpaThreads / 64];
-    __shared__ float4 acc_s[NG][TPG];
+    __shared__ float acc_s[NG][D];
 
     const size_t row = blockIdx.x;
     const int tid = threadIdx.x;
@@ -362,31 +420,39 @@ __global__ __launch_bounds__(kSdpaThreads) void sdpa_combine_kernel(CombineArgs 
     __syncthreads();
     lsum = red_s[0] + red_s[1] + red_s[2] + red_s[3];
 
-    // weighted sum of the partial rows
-    const int grp = tid / TPG, d4 = (tid % TPG) * 4;
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    const float* po = A.part_o + row * A.S * D;
-    for (int s = grp; s < A.S; s += NG) {
-        const float w = w_s[s];
-        if (w == 0.f) continue;
-        const float4 o = *reinterpret_cast<const float4*>(po + (size_t)s * D + d4);
-        acc.x = fmaf(w, o.x, acc.x); acc.y = fmaf(w, o.y, acc.y);
-        acc.z = fmaf(w, o.z, acc.z); acc.w = fmaf(w, o.w, acc.w);
-    }
-    acc_s[grp][tid % TPG] = acc;
-    __syncthreads();
-    if (tid < TPG) {
-        float4 r = acc_s[0][tid];
+    // weighted sum of the partial rows: group grp takes splits grp, grp + NG, ...
+    const int grp = tid / TPG, d8 = (tid % TPG) * 8;
+    float acc[8];
 #pragma unroll
-        for (int gI = 1; gI < NG; ++gI) {
-            const float4 o = acc_s[gI][tid];
-            r.x += o.x; r.y += o.y; r.z += o.z; r.w += o.w;
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    const uint16_t* po = A.part_o + row * A.S * D + d8;
+    for (int s0 = grp; s0 < A.S; s0 += NG * UNROLL) {
+        u32x4_t raw[UNROLL];
+        float w[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int s = s0 + u * NG;
+            w[u] = s < A.S ? w_s[s] : 0.f;
+            raw[u] = u32x4_t{0u, 0u, 0u, 0u};
+            if (w[u] != 0.f) raw[u] = *reinterpret_cast<const u32x4_t*>(po + (size_t)s * D);   // empty splits hold no data
         }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                acc[2 * e] = fmaf(w[u], Tag::to_f32((uint16_t)(raw[u][e] & 0xffffu)), acc[2 * e]);
+                acc[2 * e + 1] = fmaf(w[u], Tag::to_f32((uint16_t)(raw[u][e] >> 16)), acc[2 * e + 1]);
+            }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc_s[grp][d8 + e] = acc[e];
+    __syncthreads();
+    for (int d = tid; d < D; d += kSdpaThreads) {
+        float r = 0.f;
+#pragma unroll
+        for (int gI = 0; gI < NG; ++gI) r += acc_s[gI][d];
         const float inv = lsum == 0.f ? 1.f : 1.f / lsum;   // divide unless the sum is 0 (DFlashKernels.swift:711)
-        uint2 pk;
-        pk.x = (uint32_t)Tag::cvt(r.x * inv) | ((uint32_t)Tag::cvt(r.y * inv) << 16);
-        pk.y = (uint32_t)Tag::cvt(r.z * inv) | ((uint32_t)Tag::cvt(r.w * inv) << 16);
-        *reinterpret_cast<uint2*>(A.out + row * D + tid * 4) = pk;
+        A.out[row * D + d] = Tag::cvt(r * inv);
     }
     if (tid == 0 && A.lse) A.lse[row] = (mx + log2f(lsum)) * 0.6931471805599453f;
 }
@@ -406,7 +472,7 @@ static int choose_splits(int B, int Hk, int groups_per_kv, int N) {
 
 static size_t ws_layout(int B, int Hq, int S, int D, size_t* off_m, size_t* off_l) {
     const size_t rows = (size_t)B * Hq * kM;
-    size_t o = rows * S * D * sizeof(float);
+    size_t o = rows * S * D * sizeof(uint16_t);
     o = (o + 255) & ~(size_t)255;
     *off_m = o;
     o += rows * S * sizeof(float);
@@ -426,9 +492,15 @@ static int launch_sdpa(hipStream_t st, const SdpaArgs& A, const CombineArgs& C, 
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::BYTES);
     DFLASH_HIP_TRY(attr_rc);
     dim3 grid(A.S, A.Hk * A.groups_per_kv, B);
-    hipLaunchKernelGGL(kern, grid, dim3(kSdpaThreads), L::BYTES, st, A);
+    {
+        LaunchBracket br(DFLASH_KERNEL_SDPA_PARTIAL, st);
+        hipLaunchKernelGGL(kern, grid, dim3(kSdpaThreads), L::BYTES, st, A);
+    }
     DFLASH_HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL((sdpa_combine_kernel<Tag, D>), dim3(B * A.Hq * kM), dim3(kSdpaThreads), 0, st, C);
+    {
+        LaunchBracket br(DFLASH_KERNEL_SDPA_COMBINE, st);
+        hipLaunchKernelGGL((sdpa_combine_kernel<Tag, D>), dim3(B * A.Hq * kM), dim3(kSdpaThreads), 0, st, C);
+    }
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
 }
@@ -461,6 +533,7 @@ extern "C" int dflash_sdpa_block_causal(void* stream, const void* q, const void*
     DFLASH_SUPPORTED(Hq % Hk == 0, "sdpa: Hq=%d is not a multiple of Hk=%d", Hq, Hk);
     DFLASH_REQUIRE(N >= M, "sdpa: N=%d must include the %d block tokens", N, M);
     DFLASH_REQUIRE(kv_head_stride >= (int64_t)N * D, "sdpa: kv_head_stride smaller than N*D");
+    DFLASH_REQUIRE((int64_t)N * D * 2 < (1LL << 32), "sdpa: one KV head of %d keys exceeds the 4 GiB the kernel addresses", N);
     DFLASH_REQUIRE(kv_batch_stride >= (int64_t)(Hk - 1) * kv_head_stride + (int64_t)N * D, "sdpa: kv_batch_stride too small");
     DFLASH_REQUIRE(kv_head_stride % 8 == 0 && kv_batch_stride % 8 == 0, "sdpa: kv strides must be multiples of 8 elements");
     DFLASH_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) % 16 == 0, "sdpa: q/k/v/out must be 16-byte aligned");
@@ -476,7 +549,7 @@ extern "C" int dflash_sdpa_block_causal(void* stream, const void* q, const void*
 
     SdpaArgs A;
     A.q = (const uint16_t*)q; A.k = (const uint16_t*)k; A.v = (const uint16_t*)v;
-    A.part_o = (float*)workspace;
+    A.part_o = (uint16_t*)workspace;
     A.part_m = (float*)((char*)workspace + om);
     A.part_l = (float*)((char*)workspace + ol);
     A.kv_len_dev = kv_len_dev;

@@ -106,19 +106,20 @@ def test_kv_append_bit_exact(gpu_lib):
     lib = _lib.load()
     p = lambda t: C.c_void_p(t.data_ptr())
     assert lib.dflash_kv_append(None, p(kc), p(vc), p(kn), p(vn), B, Hk, M, D, 2, Hk * cap * D, cap * D, 100, None,
-                                cap) == 0
+                                cap, None) == 0
     k0[:, :, 100:116] = kn
     v0[:, :, 100:116] = vn
     assert torch.equal(kc, k0) and torch.equal(vc, v0)
     # offset on the device
     od = torch.tensor([250], dtype=torch.int32, device="cuda")
+    nl = torch.zeros(1, dtype=torch.int32, device="cuda")
     assert lib.dflash_kv_append(None, p(kc), p(vc), p(kn), p(vn), B, Hk, M, D, 2, Hk * cap * D, cap * D, 0, p(od),
-                                cap) == 0
+                                cap, p(nl)) == 0
     k0[:, :, 250:266] = kn
-    assert torch.equal(kc, k0)
+    assert torch.equal(kc, k0) and int(nl) == 266
     # rows outside the capacity are refused on the host
     assert lib.dflash_kv_append(None, p(kc), p(vc), p(kn), p(vn), B, Hk, M, D, 2, Hk * cap * D, cap * D, 290, None,
-                                cap) == _lib.INVALID
+                                cap, None) == _lib.INVALID
 
 
 def _forward_into_cache(cache, d, qkv, K):
