@@ -72,13 +72,14 @@ struct SdpaArgs {
     const uint16_t* q;
     const uint16_t* k;
     const uint16_t* v;
-    uint16_t* part_o;   // [B*Hq*16, S, D]  unnormalised partial O in the input type (DFlashKernels.swift:647)
+    uint16_t* part_o;   // [S, B*Hq*16, D]  unnormalised partial O in the input type (DFlashKernels.swift:647)
     float* part_m;   // [B*Hq*16, S]   running max, log2 units
     float* part_l;   // [B*Hq*16, S]   sum of exp2
     const int32_t* kv_len_dev;
     int64_t kv_batch_stride, kv_head_stride;
     float scale_log2;   // scale * log2(e)
     int Hq, Hk, G, N, S, groups_per_kv;
+    int rows_total;     // B*Hq*16
 };
 
 // LDS plan of the partial kernel.  A stage holds one tile of kBN keys: the K rows
@@ -182,31 +183,49 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
 
     // ---- asynchronous tile loads ------------------------------------------------
     // Load instruction j of this wave covers rows (4*j + wave) * RPI .. + RPI - 1 of the tile.
+    // The per-lane part of each address (row within the tile, swizzled piece) is fixed, so it is
+    // computed once; a tile that lies entirely inside the sequence only moves the scalar base.
     const int ld_rsub = lane / L::CPR;           // row within the instruction's row group
     const int ld_pos = lane % L::CPR;            // 16-byte slot this lane fills
+    uint32_t ld_off_k[L::LPW], ld_off_v[L::LPW];
+#pragma unroll
+    for (int j = 0; j < L::LPW; ++j) {
+        const int row = (4 * j + wave) * L::RPI + ld_rsub;
+        ld_off_k[j] = (uint32_t)row * L::ROWB + (uint32_t)((ld_pos ^ (row & 15)) * 16);
+        ld_off_v[j] = (uint32_t)row * L::ROWB + (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
+    }
     auto issue_tile = [&](int t) {
         const uint32_t stage_lds = smem_lds + ((t - t_begin) % kStages) * L::STAGE;
         const int key0 = t * kBN;
+        if (key0 + kBN <= Nb) {                  // uniform: whole tile in range
+            const unsigned char* kt = kbase + (size_t)key0 * L::ROWB;
+            const unsigned char* vt = vbase + (size_t)key0 * L::ROWB;
 #pragma unroll
-        for (int j = 0; j < L::LPW; ++j) {
-            const int rg = (4 * j + wave) * L::RPI;
-            const int row = rg + ld_rsub;
-            int key = key0 + row;
-            key = key < Nb ? key : Nb - 1;
-            const uint32_t goff_k = (uint32_t)key * L::ROWB + (uint32_t)((ld_pos ^ (row & 15)) * 16);
-            const uint32_t goff_v = (uint32_t)key * L::ROWB + (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
-            async_load_16B(kbase, goff_k, stage_lds + rg * L::ROWB);
-            async_load_16B(vbase, goff_v, stage_lds + L::K_BYTES + rg * L::ROWB);
+            for (int j = 0; j < L::LPW; ++j) {
+                const int rg = (4 * j + wave) * L::RPI;
+                async_load_16B(kt, ld_off_k[j], stage_lds + rg * L::ROWB);
+                async_load_16B(vt, ld_off_v[j], stage_lds + L::K_BYTES + rg * L::ROWB);
+            }
+        } else {                                 // last tile: rows past the end re-read the last key (masked later)
+#pragma unroll
+            for (int j = 0; j < L::LPW; ++j) {
+                const int rg = (4 * j + wave) * L::RPI;
+                const int row = rg + ld_rsub;
+                int key = key0 + row;
+                key = key < Nb ? key : Nb - 1;
+                const uint32_t goff_k = (uint32_t)key * L::ROWB + (uint32_t)((ld_pos ^ (row & 15)) * 16);
+                const uint32_t goff_v = (uint32_t)key * L::ROWB + (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
+                async_load_16B(kbase, goff_k, stage_lds + rg * L::ROWB);
+                async_load_16B(vbase, goff_v, stage_lds + L::K_BYTES + rg * L::ROWB);
+            }
         }
     };
     constexpr int LD_PER_TILE = 2 * L::LPW;      // vmcnt events per tile and wave
 
-    // The first kStages-1 tiles go out before anything else so that Q and the tiles share one
-    // memory round trip.  (Older loads retire first, so the compiler's own vmcnt waits for Q,
-    // which count only its loads, are conservative and stay correct.)
-#pragma unroll
-    for (int i = 0; i < kStages - 1; ++i)
-        if (t_begin + i < t_end) issue_tile(t_begin + i);
+    // Tile 0 goes out first, then Q; both are awaited together (one memory round trip), and only
+    // then the rest of the prefetch window is issued, so the first multiply does not wait for
+    // kStages-1 tiles from every CU at once.
+    issue_tile(t_begin);
 
     // ---- Q as B operands: column c = query row, k-elements 16*s + 8h .. +7 ----
     vec8 qreg[KSTEPS];
@@ -223,6 +242,9 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
     // tile loads, so a Q wait left to it lands on the first MFMA INSIDE the loop as a full
     // vmcnt(0) drain per tile, which serialises loading and computing.
     wait_vmcnt<0>();
+#pragma unroll
+    for (int i = 1; i < kStages - 1; ++i)
+        if (t_begin + i < t_end) issue_tile(t_begin + i);
 
     f32x16_t oacc[DB];
 #pragma unroll
@@ -254,15 +276,20 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
             const unsigned char* vs = ks + L::K_BYTES;
 
             // ---- S^T = K Q^T for the tile's 32 keys ----
-            f32x16_t sacc;
+            // Two accumulators: a dependent MFMA waits out the full pipeline latency of its
+            // predecessor, two interleaved chains keep the matrix pipe issuing every slot.
+            f32x16_t sacc, sacc1;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) sacc[v] = 0.f;
+            for (int v = 0; v < 16; ++v) { sacc[v] = 0.f; sacc1[v] = 0.f; }
             vec8 ka[KSTEPS];
 #pragma unroll
             for (int s = 0; s < KSTEPS; ++s)
                 ka[s] = *reinterpret_cast<const vec8*>(ks + k_rd + (((2 * s + h) ^ k_sw) * 16));
 #pragma unroll
-            for (int s = 0; s < KSTEPS; ++s) sacc = Tag::mfma(ka[s], qreg[s], sacc);
+            for (int s = 0; s < KSTEPS; s += 2) {
+                sacc = Tag::mfma(ka[s], qreg[s], sacc);
+                sacc1 = Tag::mfma(ka[s + 1], qreg[s + 1], sacc1);
+            }
             // Issue order for the block above: half of the operand reads up front, then one read per
             // MFMA, so the LDS latency hides behind the matrix pipe instead of stalling every MFMA.
             __builtin_amdgcn_sched_group_barrier(0x100, KSTEPS / 2, 0);
@@ -272,6 +299,8 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             }
             __builtin_amdgcn_sched_group_barrier(0x008, KSTEPS / 2, 0);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) sacc[v] += sacc1[v];
 
             // ---- scale, causal mask, online softmax (log2 domain) ----
             const int key0 = t * kBN;
@@ -369,7 +398,7 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
                 uint2 pk;
                 pk.x = (uint32_t)Tag::cvt(o[u].x) | ((uint32_t)Tag::cvt(o[u].y) << 16);
                 pk.y = (uint32_t)Tag::cvt(o[u].z) | ((uint32_t)Tag::cvt(o[u].w) << 16);
-                if (r < rows) *reinterpret_cast<uint2*>(A.part_o + ((rid0 + r) * A.S + split) * D + d) = pk;
+                if (r < rows) *reinterpret_cast<uint2*>(A.part_o + ((size_t)split * A.rows_total + rid0 + r) * D + d) = pk;
             }
         }
     }
@@ -425,7 +454,7 @@ __global__ __launch_bounds__(kSdpaThreads) void sdpa_combine_kernel(CombineArgs 
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-    const uint16_t* po = A.part_o + row * A.S * D + d8;
+    const uint16_t* po = A.part_o + row * D + d8;
     for (int s0 = grp; s0 < A.S; s0 += NG * UNROLL) {
         u32x4_t raw[UNROLL];
         float w[UNROLL];
@@ -434,7 +463,7 @@ __global__ __launch_bounds__(kSdpaThreads) void sdpa_combine_kernel(CombineArgs 
             const int s = s0 + u * NG;
             w[u] = s < A.S ? w_s[s] : 0.f;
             raw[u] = u32x4_t{0u, 0u, 0u, 0u};
-            if (w[u] != 0.f) raw[u] = *reinterpret_cast<const u32x4_t*>(po + (size_t)s * D);   // empty splits hold no data
+            if (w[u] != 0.f) raw[u] = *reinterpret_cast<const u32x4_t*>(po + (size_t)s * gridDim.x * D);   // empty splits hold no data
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
@@ -555,7 +584,7 @@ extern "C" int dflash_sdpa_block_causal(void* stream, const void* q, const void*
     A.kv_len_dev = kv_len_dev;
     A.kv_batch_stride = kv_batch_stride; A.kv_head_stride = kv_head_stride;
     A.scale_log2 = scale * 1.4426950408889634f;
-    A.Hq = Hq; A.Hk = Hk; A.G = G; A.N = N; A.S = S; A.groups_per_kv = groups;
+    A.Hq = Hq; A.Hk = Hk; A.G = G; A.N = N; A.S = S; A.groups_per_kv = groups; A.rows_total = B * Hq * kM;
     CombineArgs C;
     C.part_o = A.part_o; C.part_m = A.part_m; C.part_l = A.part_l;
     C.out = (uint16_t*)out; C.lse = lse; C.S = S;
