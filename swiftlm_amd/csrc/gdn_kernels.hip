@@ -245,12 +245,21 @@ constexpr int kGdnChunk = 16;  // steps staged in LDS at a time
 // LPR lanes share one state row; each keeps DK/LPR channels as float4 pieces
 // interleaved across the group (piece c of lane j covers channels
 // c*4*LPR + 4j .. +3) so that state loads and stores are fully coalesced.
-// The two row dot products (S'k for the innovation, S'q for the read-out) are
-// reduced together with DPP adds inside the 16-lane row; the read-out uses
+// Three row dot products are reduced together with DPP adds inside the 16-lane
+// row: S'k for the innovation, S'q for the read-out and k.q, because
 //   y = (S' + delta (x) k) q = S'q + delta * (k.q),
-// so the second reduction does not wait for delta.
+// so only S'k sits on the step-to-step critical path.  The kernel is bound by
+// the latency of that serial chain (T dependent steps), not by bandwidth: each
+// step's operands are therefore fetched from LDS one step ahead, and the dot
+// products run as two half-length chains.
 // Grid: x = Dv tiles of ROWS = 256/LPR rows, y = b*Hv + hv.
-template <typename StateT, bool VEC_G, int DK, int LPR>
+template <int CH> struct GdnStepOps {
+    float4 k[CH], q[CH], g[CH];
+    float gs, v, beta, kq;
+    int on;
+};
+
+template <typename StateT, bool VEC_G, bool HAS_MASK, int DK, int LPR>
 __global__ __launch_bounds__(kThreads) void gated_delta_tape_kernel(GdnArgs A) {
     constexpr int ROWS = kThreads / LPR;
     constexpr int CH = DK / (4 * LPR);
@@ -284,6 +293,21 @@ __global__ __launch_bounds__(kThreads) void gated_delta_tape_kernel(GdnArgs A) {
 #pragma unroll
     for (int c = 0; c < CH; ++c) s[c] = load4(s_in + c * 4 * LPR + 4 * j);
 
+    auto fetch = [&](int t, GdnStepOps<CH>& o) {
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int d = c * 4 * LPR + 4 * j;
+            o.k[c] = *reinterpret_cast<const float4*>(&k_s[t][d]);
+            o.q[c] = *reinterpret_cast<const float4*>(&q_s[t][d]);
+            if (VEC_G) o.g[c] = *reinterpret_cast<const float4*>(&g_s[t][d]);
+        }
+        o.gs = VEC_G ? 1.f : g_s[0][t];
+        o.v = v_s[t][rloc];
+        o.beta = beta_s[t];
+        o.kq = kq_s[t];
+        o.on = HAS_MASK ? on_s[t] : 1;
+    };
+
     for (int t0 = 0; t0 < A.T; t0 += TC) {
         const int tc = (A.T - t0) < TC ? (A.T - t0) : TC;
         if (t0) __syncthreads();
@@ -304,10 +328,11 @@ __global__ __launch_bounds__(kThreads) void gated_delta_tape_kernel(GdnArgs A) {
             const size_t bt = (size_t)b * A.T + t0 + tid;
             if (!VEC_G) g_s[0][tid] = load1_rt(A.g, A.in_dtype, bt * A.Hv + hv);
             beta_s[tid] = load1_rt(A.beta, A.in_dtype, bt * A.Hv + hv);
-            on_s[tid] = A.mask ? (int)mask_on(A.mask, A.mask_dtype, (int)bt) : 1;
+            if (HAS_MASK) on_s[tid] = (int)mask_on(A.mask, A.mask_dtype, (int)bt);
         }
         __syncthreads();
-        // k.q per step: 16 lanes per step, 16 steps per pass of the workgroup
+
+        // k.q per step (one value per head and step): 16 lanes per step
         for (int t = tid / 16; t < tc; t += kThreads / 16) {
             float acc = 0.f;
             for (int d = tid % 16; d < DK; d += 16) acc = fmaf(k_s[t][d], q_s[t][d], acc);
@@ -316,33 +341,28 @@ __global__ __launch_bounds__(kThreads) void gated_delta_tape_kernel(GdnArgs A) {
         }
         __syncthreads();
 
-        // ---- serial steps ----
-        for (int t = 0; t < tc; ++t) {
+        // ---- serial steps, operands one step ahead (two operand sets, no register copies) ----
+        auto step = [&](int t, const GdnStepOps<CH>& cur) {
             float yv = 0.f, delta = 0.f;
-            if (on_s[t]) {                            // uniform across the workgroup
-                float sk = 0.f, sq = 0.f;
+            if (!HAS_MASK || cur.on) {                // uniform across the workgroup
+                float sk0 = 0.f, sk1 = 0.f, sq0 = 0.f, sq1 = 0.f;
 #pragma unroll
                 for (int c = 0; c < CH; ++c) {
-                    const int d = c * 4 * LPR + 4 * j;
-                    const float4 k4 = *reinterpret_cast<const float4*>(&k_s[t][d]);
-                    const float4 q4 = *reinterpret_cast<const float4*>(&q_s[t][d]);
-                    float4 g4;
-                    if (VEC_G) g4 = *reinterpret_cast<const float4*>(&g_s[t][d]);
-                    else { const float gs = g_s[0][t]; g4 = make_float4(gs, gs, gs, gs); }
+                    const float4 k4 = cur.k[c], q4 = cur.q[c];
+                    const float4 g4 = VEC_G ? cur.g[c] : make_float4(cur.gs, cur.gs, cur.gs, cur.gs);
                     s[c].x *= g4.x; s[c].y *= g4.y; s[c].z *= g4.z; s[c].w *= g4.w;
-                    sk = fmaf(s[c].x, k4.x, sk); sk = fmaf(s[c].y, k4.y, sk);
-                    sk = fmaf(s[c].z, k4.z, sk); sk = fmaf(s[c].w, k4.w, sk);
-                    sq = fmaf(s[c].x, q4.x, sq); sq = fmaf(s[c].y, q4.y, sq);
-                    sq = fmaf(s[c].z, q4.z, sq); sq = fmaf(s[c].w, q4.w, sq);
+                    sk0 = fmaf(s[c].x, k4.x, sk0); sk1 = fmaf(s[c].y, k4.y, sk1);
+                    sk0 = fmaf(s[c].z, k4.z, sk0); sk1 = fmaf(s[c].w, k4.w, sk1);
+                    sq0 = fmaf(s[c].x, q4.x, sq0); sq1 = fmaf(s[c].y, q4.y, sq1);
+                    sq0 = fmaf(s[c].z, q4.z, sq0); sq1 = fmaf(s[c].w, q4.w, sq1);
                 }
-                sk = group_sum<LPR>(sk);
-                sq = group_sum<LPR>(sq);
-                delta = (v_s[t][rloc] - sk) * beta_s[t];
-                yv = fmaf(delta, kq_s[t], sq);
+                const float sk = group_sum<LPR>(sk0 + sk1);
+                const float sq = group_sum<LPR>(sq0 + sq1);
+                delta = (cur.v - sk) * cur.beta;
+                yv = fmaf(delta, cur.kq, sq);
 #pragma unroll
                 for (int c = 0; c < CH; ++c) {
-                    const int d = c * 4 * LPR + 4 * j;
-                    const float4 k4 = *reinterpret_cast<const float4*>(&k_s[t][d]);
+                    const float4 k4 = cur.k[c];
                     s[c].x = requant<StateT>(fmaf(k4.x, delta, s[c].x));
                     s[c].y = requant<StateT>(fmaf(k4.y, delta, s[c].y));
                     s[c].z = requant<StateT>(fmaf(k4.z, delta, s[c].z));
@@ -350,6 +370,16 @@ __global__ __launch_bounds__(kThreads) void gated_delta_tape_kernel(GdnArgs A) {
                 }
             }
             if (j == 0) { y_s[t][rloc] = yv; t_s[t][rloc] = delta; }
+        };
+        GdnStepOps<CH> opa, opb;
+        fetch(0, opa);
+        for (int t = 0; t < tc; t += 2) {
+            if (t + 1 < tc) fetch(t + 1, opb);
+            step(t, opa);
+            if (t + 1 < tc) {
+                if (t + 2 < tc) fetch(t + 2, opa);
+                step(t + 1, opb);
+            }
         }
         __syncthreads();
         // ---- write this chunk's y and tape rows ----
@@ -376,8 +406,10 @@ static int launch_gdn_state(hipStream_t st, const GdnArgs& A, int B, int g_ndim,
     case DKV: {                                                                                        \
         dim3 grid((A.Dv + (kThreads / LPRV) - 1) / (kThreads / LPRV), B * A.Hv);                       \
         LaunchBracket br(DFLASH_KERNEL_GDN_FORWARD, st);                                               \
-        if (vec) hipLaunchKernelGGL((gated_delta_tape_kernel<StateT, true, DKV, LPRV>), grid, dim3(kThreads), 0, st, A); \
-        else hipLaunchKernelGGL((gated_delta_tape_kernel<StateT, false, DKV, LPRV>), grid, dim3(kThreads), 0, st, A);    \
+        if (vec && A.mask) hipLaunchKernelGGL((gated_delta_tape_kernel<StateT, true, true, DKV, LPRV>), grid, dim3(kThreads), 0, st, A);        \
+        else if (vec) hipLaunchKernelGGL((gated_delta_tape_kernel<StateT, true, false, DKV, LPRV>), grid, dim3(kThreads), 0, st, A);            \
+        else if (A.mask) hipLaunchKernelGGL((gated_delta_tape_kernel<StateT, false, true, DKV, LPRV>), grid, dim3(kThreads), 0, st, A);         \
+        else hipLaunchKernelGGL((gated_delta_tape_kernel<StateT, false, false, DKV, LPRV>), grid, dim3(kThreads), 0, st, A);                    \
         DFLASH_HIP_TRY(hipGetLastError());                                                             \
         return DFLASH_OK;                                                                              \
     }
