@@ -149,6 +149,27 @@ int dflash_sdpa_block_causal(void* stream,
                              const int32_t* kv_len_dev,
                              void* workspace, size_t workspace_bytes);
 
+/* The same attention with the block's K/V append fused in: the verify forward's
+ * KVCacheSimple.update (mlx-swift-lm, reached from the attention layer the
+ * reference's batchedSDPA2Pass was written for) followed by the SDPA, in one launch
+ * pair.  k_new, v_new [B, Hk, M, D] are the block's rows; they stand for keys
+ * N-M .. N-1 (per sequence: kv_len-M .. kv_len-1), are read from k_new/v_new by the
+ * attention, and are stored into those rows of k_cache/v_cache (layout as k/v
+ * above) by the same kernel, so a following call finds them in the cache.  N must
+ * not exceed the cache's capacity in rows.  cache_len_dev (NULL, or device
+ * int32[B]) counts the rows ALREADY in the cache, block excluded, i.e. the cache
+ * offset the accept kernel maintains; sequence b then has cache_len_dev[b] + M keys,
+ * which must not exceed N.
+ * ---------------------------------------------------------------------- */
+int dflash_sdpa_block_causal_append(void* stream,
+                                    const void* q, void* k_cache, void* v_cache,
+                                    const void* k_new, const void* v_new,
+                                    void* out, float* lse, int dtype, float scale,
+                                    int B, int Hq, int Hk, int M, int N, int D,
+                                    int64_t kv_batch_stride, int64_t kv_head_stride,
+                                    const int32_t* cache_len_dev,
+                                    void* workspace, size_t workspace_bytes);
+
 /* ------------------------------------------------------------------------
  * Acceptance.  dflash_match_acceptance_length replaces
  * DFlashRuntime.matchAcceptanceLength (Sources/DFlash/DFlashRuntime.swift:

@@ -72,6 +72,10 @@ struct SdpaArgs {
     const uint16_t* q;
     const uint16_t* k;
     const uint16_t* v;
+    const uint16_t* k_new;   // [B,Hk,16,D] rows standing for keys Nb-16 .. Nb-1, or null
+    const uint16_t* v_new;
+    uint16_t* k_cache;       // where the fused append stores those rows (== k, v), or null
+    uint16_t* v_cache;
     uint16_t* part_o;   // [S, B*Hq*16, D]  unnormalised partial O in the input type (DFlashKernels.swift:647)
     float* part_m;   // [B*Hq*16, S]   running max, log2 units
     float* part_l;   // [B*Hq*16, S]   sum of exp2
@@ -80,6 +84,7 @@ struct SdpaArgs {
     float scale_log2;   // scale * log2(e)
     int Hq, Hk, G, N, S, groups_per_kv;
     int rows_total;     // B*Hq*16
+    int len_bias;       // added to kv_len_dev[b]: 0, or 16 when the device count excludes the block
 };
 
 // LDS plan of the partial kernel.  A stage holds one tile of kBN keys: the K rows
@@ -112,6 +117,22 @@ __device__ __forceinline__ void async_load_16B(const unsigned char* gbase, uint3
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(goff), "s"(gbase), "s"(lds_base)
+                 : "memory", "m0");
+}
+
+// Tells the compiler a wave-uniform pointer is uniform (inline-assembly "s" operands need SGPRs).
+__device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char* p) {
+    const uint64_t u = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
+    return (const unsigned char*)(((uint64_t)hi << 32) | lo);
+}
+
+// Same, with a full per-lane 64-bit address (rows that come from different buffers).
+__device__ __forceinline__ void async_load_16B_addr(const unsigned char* gptr, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"((uint64_t)gptr), "s"(lds_base)
                  : "memory", "m0");
 }
 
@@ -154,7 +175,7 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
     const int b = blockIdx.z;
     const int hcount = (A.G - hg0) < kHeadsPerWG ? (A.G - hg0) : kHeadsPerWG;
 
-    int Nb = A.kv_len_dev ? A.kv_len_dev[b] : A.N;
+    int Nb = A.kv_len_dev ? A.kv_len_dev[b] + A.len_bias : A.N;
     Nb = Nb < kM ? kM : (Nb > A.N ? A.N : Nb);
     const int nt = (Nb + kBN - 1) / kBN;
     const int t_begin = (int)(((long)split * nt) / A.S);
@@ -168,6 +189,26 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
     const int qi = c & 15;
     const size_t row_id = ((size_t)b * A.Hq + hq) * kM + qi;   // valid only when row_valid
 
+    const unsigned char* kbase = reinterpret_cast<const unsigned char*>(A.k) +
+                                 ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
+    const unsigned char* vbase = reinterpret_cast<const unsigned char*>(A.v) +
+                                 ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
+
+    // Fused append: keys Nb-16 .. Nb-1 are read from k_new / v_new, and one workgroup per KV head
+    // stores them into the cache rows they stand for.
+    const bool fused = A.k_new != nullptr;
+    const int cache_rows = fused ? Nb - kM : Nb;       // keys below this index are read from the cache
+    const unsigned char* knew = reinterpret_cast<const unsigned char*>(A.k_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
+    const unsigned char* vnew = reinterpret_cast<const unsigned char*>(A.v_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
+    if (fused && A.k_cache && split == 0 && hg0 == 0) {
+        const size_t head = ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2 + (size_t)cache_rows * L::ROWB;
+        u32x4_t* kd = reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.k_cache) + head);
+        u32x4_t* vd = reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.v_cache) + head);
+        const u32x4_t* ksrc = reinterpret_cast<const u32x4_t*>(knew);
+        const u32x4_t* vsrc = reinterpret_cast<const u32x4_t*>(vnew);
+        for (int i = tid; i < kM * L::CPR; i += kSdpaThreads) { kd[i] = ksrc[i]; vd[i] = vsrc[i]; }
+    }
+
     if (t_begin >= t_end) {   // empty split: tell the combine kernel to ignore it
         if (row_valid && h == 0) {
             A.part_m[row_id * A.S + split] = -INFINITY;
@@ -175,11 +216,6 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
         }
         return;
     }
-
-    const unsigned char* kbase = reinterpret_cast<const unsigned char*>(A.k) +
-                                 ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
-    const unsigned char* vbase = reinterpret_cast<const unsigned char*>(A.v) +
-                                 ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
 
     // ---- asynchronous tile loads ------------------------------------------------
     // Load instruction j of this wave covers rows (4*j + wave) * RPI .. + RPI - 1 of the tile.
@@ -197,26 +233,32 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
     auto issue_tile = [&](int t) {
         const uint32_t stage_lds = smem_lds + ((t - t_begin) % kStages) * L::STAGE;
         const int key0 = t * kBN;
-        if (key0 + kBN <= Nb) {                  // uniform: whole tile in range
-            const unsigned char* kt = kbase + (size_t)key0 * L::ROWB;
-            const unsigned char* vt = vbase + (size_t)key0 * L::ROWB;
+        if (key0 + kBN <= cache_rows) {          // uniform: whole tile comes from the cache
+            const unsigned char* kt = uniform_ptr(kbase + (size_t)key0 * L::ROWB);
+            const unsigned char* vt = uniform_ptr(vbase + (size_t)key0 * L::ROWB);
 #pragma unroll
             for (int j = 0; j < L::LPW; ++j) {
                 const int rg = (4 * j + wave) * L::RPI;
                 async_load_16B(kt, ld_off_k[j], stage_lds + rg * L::ROWB);
                 async_load_16B(vt, ld_off_v[j], stage_lds + L::K_BYTES + rg * L::ROWB);
             }
-        } else {                                 // last tile: rows past the end re-read the last key (masked later)
+        } else {
+            // Tail tile: rows past the end re-read the last key (masked later); with a fused append
+            // the block's own 16 rows are taken from k_new / v_new instead of the cache.
 #pragma unroll
             for (int j = 0; j < L::LPW; ++j) {
                 const int rg = (4 * j + wave) * L::RPI;
                 const int row = rg + ld_rsub;
                 int key = key0 + row;
                 key = key < Nb ? key : Nb - 1;
-                const uint32_t goff_k = (uint32_t)key * L::ROWB + (uint32_t)((ld_pos ^ (row & 15)) * 16);
-                const uint32_t goff_v = (uint32_t)key * L::ROWB + (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
-                async_load_16B(kbase, goff_k, stage_lds + rg * L::ROWB);
-                async_load_16B(vbase, goff_v, stage_lds + L::K_BYTES + rg * L::ROWB);
+                const uint32_t pk = (uint32_t)((ld_pos ^ (row & 15)) * 16);
+                const uint32_t pv = (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
+                const unsigned char* ksrc = key < cache_rows ? kbase + (size_t)key * L::ROWB
+                                                              : knew + (size_t)(key - cache_rows) * L::ROWB;
+                const unsigned char* vsrc = key < cache_rows ? vbase + (size_t)key * L::ROWB
+                                                              : vnew + (size_t)(key - cache_rows) * L::ROWB;
+                async_load_16B_addr(ksrc + pk, stage_lds + rg * L::ROWB);
+                async_load_16B_addr(vsrc + pv, stage_lds + L::K_BYTES + rg * L::ROWB);
             }
         }
     };
@@ -547,10 +589,10 @@ extern "C" size_t dflash_sdpa_workspace_bytes(int B, int Hq, int Hk, int M, int 
     return ws_layout(B, Hq, choose_splits(B, Hk, groups, N), D, &om, &ol);
 }
 
-extern "C" int dflash_sdpa_block_causal(void* stream, const void* q, const void* k, const void* v, void* out,
-                                        float* lse, int dtype, float scale, int B, int Hq, int Hk, int M, int N,
-                                        int D, int64_t kv_batch_stride, int64_t kv_head_stride,
-                                        const int32_t* kv_len_dev, void* workspace, size_t workspace_bytes) {
+static int sdpa_common(void* stream, const void* q, const void* k, const void* v, const void* k_new, const void* v_new,
+                       void* k_cache, void* v_cache, void* out, float* lse, int dtype, float scale, int B, int Hq, int Hk,
+                       int M, int N, int D, int64_t kv_batch_stride, int64_t kv_head_stride, const int32_t* kv_len_dev,
+                       void* workspace, size_t workspace_bytes) {
     int rc = ensure_init();
     if (rc) return rc;
     DFLASH_REQUIRE(q && k && v && out, "sdpa: null pointer");
@@ -565,7 +607,8 @@ extern "C" int dflash_sdpa_block_causal(void* stream, const void* q, const void*
     DFLASH_REQUIRE((int64_t)N * D * 2 < (1LL << 32), "sdpa: one KV head of %d keys exceeds the 4 GiB the kernel addresses", N);
     DFLASH_REQUIRE(kv_batch_stride >= (int64_t)(Hk - 1) * kv_head_stride + (int64_t)N * D, "sdpa: kv_batch_stride too small");
     DFLASH_REQUIRE(kv_head_stride % 8 == 0 && kv_batch_stride % 8 == 0, "sdpa: kv strides must be multiples of 8 elements");
-    DFLASH_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) % 16 == 0, "sdpa: q/k/v/out must be 16-byte aligned");
+    DFLASH_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out | (uintptr_t)k_new | (uintptr_t)v_new) % 16 == 0,
+                   "sdpa: q/k/v/out must be 16-byte aligned");
     DFLASH_REQUIRE(B <= 65535 && (long)Hq * 2 <= 65535, "sdpa: batch or head count too large for one launch");
 
     const int G = Hq / Hk;
@@ -578,6 +621,8 @@ extern "C" int dflash_sdpa_block_causal(void* stream, const void* q, const void*
 
     SdpaArgs A;
     A.q = (const uint16_t*)q; A.k = (const uint16_t*)k; A.v = (const uint16_t*)v;
+    A.k_new = (const uint16_t*)k_new; A.v_new = (const uint16_t*)v_new;
+    A.k_cache = (uint16_t*)k_cache; A.v_cache = (uint16_t*)v_cache;
     A.part_o = (uint16_t*)workspace;
     A.part_m = (float*)((char*)workspace + om);
     A.part_l = (float*)((char*)workspace + ol);
@@ -585,6 +630,7 @@ extern "C" int dflash_sdpa_block_causal(void* stream, const void* q, const void*
     A.kv_batch_stride = kv_batch_stride; A.kv_head_stride = kv_head_stride;
     A.scale_log2 = scale * 1.4426950408889634f;
     A.Hq = Hq; A.Hk = Hk; A.G = G; A.N = N; A.S = S; A.groups_per_kv = groups; A.rows_total = B * Hq * kM;
+    A.len_bias = k_new ? kM : 0;
     CombineArgs C;
     C.part_o = A.part_o; C.part_m = A.part_m; C.part_l = A.part_l;
     C.out = (uint16_t*)out; C.lse = lse; C.S = S;
@@ -592,4 +638,22 @@ extern "C" int dflash_sdpa_block_causal(void* stream, const void* q, const void*
     hipStream_t st = (hipStream_t)stream;
     if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa<Bf16Tag, 256>(st, A, C, B) : launch_sdpa<Bf16Tag, 128>(st, A, C, B);
     return D == 256 ? launch_sdpa<F16Tag, 256>(st, A, C, B) : launch_sdpa<F16Tag, 128>(st, A, C, B);
+}
+
+extern "C" int dflash_sdpa_block_causal(void* stream, const void* q, const void* k, const void* v, void* out,
+                                        float* lse, int dtype, float scale, int B, int Hq, int Hk, int M, int N,
+                                        int D, int64_t kv_batch_stride, int64_t kv_head_stride,
+                                        const int32_t* kv_len_dev, void* workspace, size_t workspace_bytes) {
+    return sdpa_common(stream, q, k, v, nullptr, nullptr, nullptr, nullptr, out, lse, dtype, scale, B, Hq, Hk, M, N, D,
+                       kv_batch_stride, kv_head_stride, kv_len_dev, workspace, workspace_bytes);
+}
+
+extern "C" int dflash_sdpa_block_causal_append(void* stream, const void* q, void* k_cache, void* v_cache,
+                                               const void* k_new, const void* v_new, void* out, float* lse, int dtype,
+                                               float scale, int B, int Hq, int Hk, int M, int N, int D,
+                                               int64_t kv_batch_stride, int64_t kv_head_stride,
+                                               const int32_t* cache_len_dev, void* workspace, size_t workspace_bytes) {
+    DFLASH_REQUIRE(k_new && v_new && k_cache && v_cache, "sdpa (append): null pointer");
+    return sdpa_common(stream, q, k_cache, v_cache, k_new, v_new, k_cache, v_cache, out, lse, dtype, scale, B, Hq, Hk, M,
+                       N, D, kv_batch_stride, kv_head_stride, cache_len_dev, workspace, workspace_bytes);
 }

@@ -181,6 +181,51 @@ class DFlashKernels:
         return (out, lse) if return_lse else out
 
     @staticmethod
+    def batched_sdpa_2pass_append(queries: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                                  k_new: torch.Tensor, v_new: torch.Tensor, scale: float, n_keys: int, *,
+                                  return_lse: bool = False, cache_len: Optional[torch.Tensor] = None,
+                                  workspace: Optional[torch.Tensor] = None):
+        """The verify block's attention with its KV append fused in (one launch pair instead of
+        ``KVCacheSimple.update`` + ``batchedSDPA2Pass``).  ``k_cache``/``v_cache`` [B,Hk,capacity,D]
+        hold ``n_keys - 16`` valid rows per sequence (``cache_len[b]`` when the int32 device
+        tensor ``cache_len`` is given; ``n_keys`` is then the upper bound of cache_len + 16);
+        ``k_new``/``v_new`` [B,Hk,16,D] are the block's rows, attended as keys n_keys-16 .. n_keys-1
+        and written into those cache rows.  Returns None for unsupported shapes."""
+        _dev(queries, k_cache, v_cache, k_new, v_new, cache_len, workspace)
+        if queries.dim() != 4 or k_cache.dim() != 4 or k_cache.shape != v_cache.shape:
+            return None
+        B, Hq, M, D = queries.shape
+        Hk, cap = k_cache.shape[1], k_cache.shape[2]
+        if (k_new.shape != (B, Hk, M, D) or v_new.shape != (B, Hk, M, D) or k_cache.shape[3] != D
+                or any(t.dtype != queries.dtype for t in (k_cache, v_cache, k_new, v_new))):
+            return None
+        if not (M <= n_keys <= cap):
+            raise DFlashError(f"batched_sdpa_2pass_append: n_keys={n_keys} outside [{M}, capacity={cap}]")
+        if k_cache.stride(3) != 1 or k_cache.stride(2) != D or k_cache.stride() != v_cache.stride():
+            raise DFlashError("batched_sdpa_2pass_append: the caches must be row-contiguous and laid out alike")
+        queries, k_new, v_new = queries.contiguous(), k_new.contiguous(), v_new.contiguous()
+        lib = _lib.load()
+        need = int(lib.dflash_sdpa_workspace_bytes(B, Hq, Hk, M, n_keys, D))
+        if need == 0:
+            return None
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=queries.device)
+        out = torch.empty_like(queries)
+        lse = torch.empty((B, Hq, M), dtype=torch.float32, device=queries.device) if return_lse else None
+        try:
+            code = _code(queries)
+        except DFlashUnsupported:
+            return None
+        rc = lib.dflash_sdpa_block_causal_append(
+            _stream(), _ptr(queries), _ptr(k_cache), _ptr(v_cache), _ptr(k_new), _ptr(v_new), _ptr(out), _ptr(lse),
+            code, float(scale), B, Hq, Hk, M, int(n_keys), D, k_cache.stride(0), k_cache.stride(1), _ptr(cache_len),
+            _ptr(workspace), workspace.numel() * workspace.element_size())
+        if rc == _lib.UNSUPPORTED:
+            return None
+        _lib.check(rc, "batched_sdpa_2pass_append")
+        return (out, lse) if return_lse else out
+
+    @staticmethod
     def sdpa_fallback(queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, scale: float,
                       mask: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``sdpaFallback`` (DFlashKernels.swift:818-828) delegates to the array library's

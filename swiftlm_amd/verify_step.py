@@ -5,8 +5,8 @@ loop runs it (Sources/DFlash/DFlashRuntime.swift:484-581):
 
   1. per GatedDelta layer: forward-with-tape from the pre-verify state into a second
      state buffer (the rollback cache is armed by reference, so nothing is copied);
-     per attention layer: append the block's 16 K/V rows at the cache offset, then the
-     block-causal SDPA over offset+16 keys;
+     per attention layer: the block-causal SDPA over offset+16 keys with the append of the
+     block's 16 K/V rows at the cache offset fused in;
   2. acceptance length / commit count on the device (no host round trip);
   3. rollback: ONE batched tape-replay launch for all GatedDelta layers that reads the
      commit count from device memory and leaves a fully accepted block alone; the KV
@@ -104,9 +104,8 @@ class HybridVerifyStack:
             raise _lib.DFlashError("sdpa workspace query failed: " + _lib.last_error())
         self.workspace = torch.empty(max(ws, 256), dtype=torch.uint8, device=device)
         self.n_max = n_max
-        # device-side scalars: cache offset L, key count L+16, and the accept kernel's outputs
+        # device-side scalars: cache offset L (advanced by the accept kernel) and that kernel's outputs
         self.offset = torch.tensor([cfg.context], dtype=torch.int32, device=device)
-        self.kv_len = torch.tensor([cfg.context + T], dtype=torch.int32, device=device)
         self.accept = torch.zeros(4, dtype=torch.int32, device=device)
         # acceptance inputs of the step being enqueued, one pair per ping-pong phase
         self.verify_ids = [torch.zeros(T, dtype=torch.int32, device=device) for _ in range(2)]
@@ -142,15 +141,11 @@ class HybridVerifyStack:
             else:
                 l = self.attn[ai]; ai += 1
                 hs = cfg.capacity * cfg.D
-                rc = lib.dflash_kv_append(st, _p(l["k_cache"]), _p(l["v_cache"]), _p(l["k_new"]), _p(l["v_new"]),
-                                          1, cfg.Hkv, T, cfg.D, 2, cfg.Hkv * hs, hs, 0, _p(self.offset), cfg.capacity,
-                                          _p(self.kv_len))
-                _lib.check(rc, "kv_append")
                 note("sdpa")
-                rc = lib.dflash_sdpa_block_causal(
-                    st, _p(l["q"]), _p(l["k_cache"]), _p(l["v_cache"]), _p(l["out"]), _p(l["lse"]), _lib.BF16,
-                    self.scale, 1, cfg.Hq, cfg.Hkv, T, self.n_max, cfg.D, cfg.Hkv * hs, hs, _p(self.kv_len),
-                    _p(self.workspace), self.workspace.numel())
+                rc = lib.dflash_sdpa_block_causal_append(
+                    st, _p(l["q"]), _p(l["k_cache"]), _p(l["v_cache"]), _p(l["k_new"]), _p(l["v_new"]), _p(l["out"]),
+                    _p(l["lse"]), _lib.BF16, self.scale, 1, cfg.Hq, cfg.Hkv, T, self.n_max, cfg.D, cfg.Hkv * hs, hs,
+                    _p(self.offset), _p(self.workspace), self.workspace.numel())
                 _lib.check(rc, "sdpa_block_causal")
         # accept: commit count -> accept[1]; offset += commit count
         rc = lib.dflash_accept_commit(st, _p(self.verify_ids[ph]), _p(self.posterior[ph]), T, _p(self.offset),

@@ -156,3 +156,49 @@ def test_sdpa_unsupported_shapes_return_none(gpu_lib):
     assert K.batched_sdpa_2pass(q[0], k[0], v[0], 0.1) is None                   # ndim != 4
     with pytest.raises(DFlashUnsupported):
         K.sdpa_fallback(q64, k64, v64, 0.1)
+
+
+@pytest.mark.parametrize("cfg", [(1, 16, 2, 0, 256), (1, 16, 2, 7, 256), (2, 8, 2, 300, 128), (1, 16, 2, 4096, 256)],
+                         ids=lambda c: f"B{c[0]}_Hq{c[1]}_Hk{c[2]}_L{c[3]}_D{c[4]}")
+def test_sdpa_fused_append_equals_append_then_sdpa(gpu_lib, cfg):
+    """The fused entry must give the bytes of `append, then attend`: same O and LSE, and the
+    block's rows stored bit for bit at rows L .. L+15 of the cache, nothing else touched."""
+    from swiftlm_amd import DFlashKernels as K
+
+    B, Hq, Hk, L, D = cfg
+    q, k, v = gpu_inputs(L + 5, B, Hq, Hk, L, D)
+    cap = L + 16 + 37
+    kc = torch.full((B, Hk, cap, D), 3.0, dtype=torch.bfloat16, device="cuda")
+    vc = torch.full((B, Hk, cap, D), -3.0, dtype=torch.bfloat16, device="cuda")
+    kc[:, :, :L], vc[:, :, :L] = k[:, :, :L], v[:, :, :L]
+    k_new, v_new = k[:, :, L:].contiguous(), v[:, :, L:].contiguous()
+    scale = 1.0 / math.sqrt(D)
+    want, want_lse = K.batched_sdpa_2pass(q, k, v, scale, return_lse=True)
+    got, got_lse = K.batched_sdpa_2pass_append(q, kc, vc, k_new, v_new, scale, L + 16, return_lse=True)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want) and torch.equal(got_lse, want_lse)
+    assert torch.equal(kc[:, :, : L + 16], k) and torch.equal(vc[:, :, : L + 16], v)
+    assert bool((kc[:, :, L + 16:] == 3.0).all()) and bool((vc[:, :, L + 16:] == -3.0).all())
+    # and the next step reads them back from the cache
+    again = K.batched_sdpa_2pass(q, kc[:, :, : L + 16], vc[:, :, : L + 16], scale)
+    assert torch.equal(again, want)
+
+
+def test_sdpa_fused_append_ragged(gpu_lib):
+    from swiftlm_amd import DFlashKernels as K
+
+    B, Hq, Hk, D, cap = 3, 16, 2, 256, 700
+    Ls = [100, 333, 650]
+    q, k, v = gpu_inputs(9, B, Hq, Hk, cap - 16, D)
+    kc, vc = k.clone(), v.clone()
+    k_new = torch.stack([k[b, :, Ls[b]:Ls[b] + 16] for b in range(B)]).contiguous()
+    v_new = torch.stack([v[b, :, Ls[b]:Ls[b] + 16] for b in range(B)]).contiguous()
+    for b in range(B):                                  # poison the rows the append must fill
+        kc[b, :, Ls[b]:Ls[b] + 16] = 9.0
+        vc[b, :, Ls[b]:Ls[b] + 16] = 9.0
+    kv_len = torch.tensor([l + 16 for l in Ls], dtype=torch.int32, device="cuda")
+    cache_len = torch.tensor(Ls, dtype=torch.int32, device="cuda")
+    want = K.batched_sdpa_2pass(q, k, v, 1.0 / 16, kv_len=kv_len)
+    got = K.batched_sdpa_2pass_append(q, kc, vc, k_new, v_new, 1.0 / 16, cap, cache_len=cache_len)
+    assert torch.equal(got, want)
+    assert torch.equal(kc, k) and torch.equal(vc, v)
