@@ -129,6 +129,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="enqueue every step from the host instead of replaying graphs")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--context", type=int, default=32768)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy, the known-size kernel the rocprof byte counters are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -297,6 +299,13 @@ def main():
             "launches_timed": sdpa_launches,
         },
     }
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        result["calibration_copy_bytes"] = int(src.numel())
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg, mean_commit)
     else:

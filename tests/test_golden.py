@@ -1,0 +1,120 @@
+"""Committed fixtures (tests/golden/*.npz, written by tests/golden/make_golden.py from the
+oracle): the oracles must keep reproducing them on the CPU, and the HIP kernels must match them
+on the GPU."""
+
+import glob
+import os
+
+import numpy as np
+import pytest
+
+from oracle import c_oracle
+from oracle import dflash_oracle as O
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def load(name):
+    return dict(np.load(os.path.join(GOLD, name), allow_pickle=False))
+
+
+def gdn_files():
+    return sorted(os.path.basename(p) for p in glob.glob(os.path.join(GOLD, "gdn_*.npz")))
+
+
+def sdpa_files():
+    return sorted(os.path.basename(p) for p in glob.glob(os.path.join(GOLD, "sdpa_*.npz")))
+
+
+@pytest.mark.parametrize("name", gdn_files())
+def test_oracles_reproduce_gdn_fixture(name):
+    f = load(name)
+    mask = f["mask"] if f["mask"].size else None
+    n = int(f["n_accept"])
+    for impl in ("numpy", "c"):
+        if impl == "numpy":
+            y, S, tape = O.gated_delta_ops_with_tape(f["q"], f["k"], f["v"], f["g"], f["beta"], f["state"], mask)
+            rep = O.tape_replay_ops(f["tape"][:, :n], f["k"][:, :n], f["g"][:, :n], f["state"],
+                                    None if mask is None else mask[:, :n])
+        else:
+            y, S, tape = c_oracle.gated_delta(f["q"], f["k"], f["v"], f["g"], f["beta"], f["state"], mask)
+            rep = c_oracle.tape_replay(f["tape"][:, :n], f["k"][:, :n], f["g"][:, :n], f["state"],
+                                       None if mask is None else mask[:, :n])
+        np.testing.assert_allclose(y, f["y"], rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(S, f["state_out"], rtol=1e-4, atol=1e-6)
+        np.testing.assert_allclose(tape, f["tape"], rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(rep, f["replayed"], rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize("name", sdpa_files())
+def test_oracles_reproduce_sdpa_fixture(name):
+    f = load(name)
+    o, lse = c_oracle.sdpa_block_causal(f["q"], f["k"], f["v"], float(f["scale"]))
+    np.testing.assert_allclose(o, f["out"], rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(lse, f["lse"], rtol=1e-5, atol=1e-5)
+
+
+def test_oracle_reproduces_accept_fixture():
+    cases = load("accept_commit_cases.npz")["cases"]
+    for row in cases:
+        staged, drafted, posterior, start = int(row[0]), row[1:16], row[16:32], int(row[32])
+        r = O.accept_commit(staged, drafted, posterior, start)
+        assert [r["acceptance_len"], r["commit_count"], r["staged_next"], r["start"]] == list(row[33:37])
+        assert c_oracle.match_acceptance_length(drafted, posterior[:15]) == row[33]
+
+
+# ------------------------------------------------------------------ GPU ------
+
+
+def _dev(a, dt):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda", dt)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", gdn_files())
+def test_hip_matches_gdn_fixture(gpu_lib, name):
+    import torch
+
+    from swiftlm_amd import DFlashKernels as K
+
+    f = load(name)
+    dt = {"f32": torch.float32, "bf16": torch.bfloat16}[str(f["in_dtype"])]
+    mask = _dev(f["mask"], torch.float32) if f["mask"].size else None
+    n = int(f["n_accept"])
+    q, k, v, g, beta = (_dev(f[x], dt) for x in ("q", "k", "v", "g", "beta"))
+    s0 = _dev(f["state"], torch.float32)
+    y, S, tape = K.gated_delta_kernel_with_tape(q, k, v, g, beta, s0, mask)
+    rep = K.tape_replay_kernel(tape[:, :n], k[:, :n], g[:, :n], s0, None if mask is None else mask[:, :n])
+    h = lambda t: t.float().cpu().numpy()
+    ytol = dict(rtol=1e-4, atol=1e-5) if dt == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    np.testing.assert_allclose(h(y), f["y"], **ytol)
+    np.testing.assert_allclose(h(S), f["state_out"], rtol=1e-4, atol=1e-6)
+    np.testing.assert_allclose(h(tape), f["tape"], rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(h(rep), f["replayed"], rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sdpa_files())
+def test_hip_matches_sdpa_fixture(gpu_lib, name):
+    import torch
+
+    from swiftlm_amd import DFlashKernels as K
+
+    f = load(name)
+    out, lse = K.batched_sdpa_2pass(_dev(f["q"], torch.bfloat16), _dev(f["k"], torch.bfloat16),
+                                    _dev(f["v"], torch.bfloat16), float(f["scale"]), return_lse=True)
+    np.testing.assert_allclose(out.float().cpu().numpy(), f["out"], rtol=2e-2, atol=2e-2)
+    np.testing.assert_allclose(lse.cpu().numpy(), f["lse"], rtol=2e-3, atol=2e-3)
+
+
+@pytest.mark.gpu
+def test_hip_matches_accept_fixture(gpu_lib):
+    import torch
+
+    from swiftlm_amd import DFlashRuntime as R
+
+    for row in load("accept_commit_cases.npz")["cases"]:
+        r = R.accept_commit(torch.from_numpy(row[0:16]).cuda(), torch.from_numpy(row[16:32]).cuda(), int(row[32]))
+        assert [r.acceptance_len, r.commit_count, r.staged_first_next, r.start] == list(row[33:37])
