@@ -304,43 +304,57 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
     const int v_piece = 2 * (tg & 1) + (tq >> 1);        // 16-byte piece within a 32-channel block
     const int v_sw = 4 * tj;                             // row % 4 == tj for every row this lane reads
 
-    for (int t = t_begin; t < t_end; ++t) {
-        // tile t has landed once at most (tiles issued after it) * LD_PER_TILE loads are outstanding
-        const int ahead = (t_end - 1 - t) < (kStages - 2) ? (t_end - 1 - t) : (kStages - 2);
-        if (ahead >= 2) wait_vmcnt<2 * LD_PER_TILE>();
-        else if (ahead == 1) wait_vmcnt<LD_PER_TILE>();
-        else wait_vmcnt<0>();
-        __builtin_amdgcn_s_barrier();   // everyone's share of tile t is in LDS; everyone is done with tile t-1
-        if (t + kStages - 1 < t_end) issue_tile(t + kStages - 1);   // refills the stage tile t-1 used
+    // The tile loop is split in two levels so that NOTHING inside the hot inner loop touches the O
+    // accumulators except the MFMAs: when a row's maximum jumps (rare, see kRescaleLog2) the wave
+    // leaves the inner loop before using the tile, rescales in the cold outer block and re-enters
+    // at the same tile.  With the rescale written inside the hot loop the register allocator keeps
+    // a VGPR copy of all 128 accumulator registers and refreshes it on every iteration.
+    int t = t_begin;
+    bool resume = false;          // tile t was already awaited, announced and prefetched for
+    float m_pending = -INFINITY;
+    while (t < t_end) {
+    bool jumped = false;
+    for (; t < t_end; ++t) {
+        if (!resume) {
+            // tile t has landed once at most (tiles issued after it) * LD_PER_TILE loads are outstanding
+            const int ahead = (t_end - 1 - t) < (kStages - 2) ? (t_end - 1 - t) : (kStages - 2);
+            if (ahead >= 2) wait_vmcnt<2 * LD_PER_TILE>();
+            else if (ahead == 1) wait_vmcnt<LD_PER_TILE>();
+            else wait_vmcnt<0>();
+            __builtin_amdgcn_s_barrier();   // everyone's share of tile t is in LDS; everyone is done with tile t-1
+            if (t + kStages - 1 < t_end) issue_tile(t + kStages - 1);   // refills the stage tile t-1 used
+        }
+        resume = false;
 
         if (wave_active) {
             const unsigned char* ks = smem + ((t - t_begin) % kStages) * L::STAGE;
             const unsigned char* vs = ks + L::K_BYTES;
 
             // ---- S^T = K Q^T for the tile's 32 keys ----
-            // Two accumulators: a dependent MFMA waits out the full pipeline latency of its
-            // predecessor, two interleaved chains keep the matrix pipe issuing every slot.
+            // Two accumulators: a dependent 32x32x16 MFMA waits out the full pipeline latency of its
+            // predecessor (~2.4 issue slots), so two interleaved chains roughly halve the Q K^T time
+            // (more chains cost more accumulator read-outs than they save).  Operand reads run
+            // kQkAhead k-steps ahead of the MFMAs; sched_barrier pins that order (left alone, the
+            // scheduler issues one whole chain after the other).
+            constexpr int kQkAhead = 8;
             f32x16_t sacc, sacc1;
 #pragma unroll
             for (int v = 0; v < 16; ++v) { sacc[v] = 0.f; sacc1[v] = 0.f; }
             vec8 ka[KSTEPS];
 #pragma unroll
-            for (int s = 0; s < KSTEPS; ++s)
+            for (int s = 0; s < kQkAhead; ++s)
                 ka[s] = *reinterpret_cast<const vec8*>(ks + k_rd + (((2 * s + h) ^ k_sw) * 16));
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int s = 0; s < KSTEPS; s += 2) {
+                if (s + kQkAhead < KSTEPS) {
+                    ka[s + kQkAhead] = *reinterpret_cast<const vec8*>(ks + k_rd + (((2 * (s + kQkAhead) + h) ^ k_sw) * 16));
+                    ka[s + kQkAhead + 1] = *reinterpret_cast<const vec8*>(ks + k_rd + (((2 * (s + kQkAhead + 1) + h) ^ k_sw) * 16));
+                }
                 sacc = Tag::mfma(ka[s], qreg[s], sacc);
                 sacc1 = Tag::mfma(ka[s + 1], qreg[s + 1], sacc1);
+                __builtin_amdgcn_sched_barrier(0);
             }
-            // Issue order for the block above: half of the operand reads up front, then one read per
-            // MFMA, so the LDS latency hides behind the matrix pipe instead of stalling every MFMA.
-            __builtin_amdgcn_sched_group_barrier(0x100, KSTEPS / 2, 0);
-#pragma unroll
-            for (int s = 0; s < KSTEPS / 2; ++s) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, KSTEPS / 2, 0);
 #pragma unroll
             for (int v = 0; v < 16; ++v) sacc[v] += sacc1[v];
 
@@ -364,10 +378,13 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
             // exceeds it by more than kRescaleLog2 (P then stays below 2^kRescaleLog2, harmless in
             // fp32/bf16), so the 128 accumulator registers are rarely touched by the softmax.
             const bool bump = mloc > m_run + kRescaleLog2;      // also true for the first finite maximum
-            const float m_new = bump ? mloc : m_run;
+            if (__builtin_amdgcn_ballot_w64(bump && m_run != -INFINITY) != 0) {
+                m_pending = mloc;                               // accumulators hold data: rescale first
+                jumped = true;
+                break;
+            }
+            const float m_new = bump ? mloc : m_run;            // a bump here starts from an empty row
             const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = bump ? fast_exp2(m_run - m_safe) : 1.f;
-            const bool rescale = bump && m_run != -INFINITY;    // nothing accumulated yet otherwise
             m_run = m_new;
             float psum = 0.f;
 #pragma unroll
@@ -376,13 +393,7 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
                 sacc[v] = p;
                 psum += p;
             }
-            l_run = l_run * alpha + psum;
-            if (__builtin_amdgcn_ballot_w64(rescale) != 0) {
-#pragma unroll
-                for (int i = 0; i < DB; ++i)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
-            }
+            l_run += psum;
 
             // ---- O^T += V^T P^T ----
             // MFMA ksub feeds accumulator registers 8*ksub .. 8*ksub+7, i.e. keys
@@ -405,6 +416,18 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
                 }
             }
         }
+    }
+    if (jumped) {
+        const bool bump = m_pending > m_run + kRescaleLog2;
+        const float alpha = (bump && m_run != -INFINITY) ? fast_exp2(m_run - m_pending) : 1.f;
+        if (bump) m_run = m_pending;
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < DB; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
+        resume = true;
+    }
     }
     __syncthreads();          // the tile buffers are free for the epilogue
 
