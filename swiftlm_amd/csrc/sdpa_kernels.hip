@@ -304,131 +304,171 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
     const int v_piece = 2 * (tg & 1) + (tq >> 1);        // 16-byte piece within a 32-channel block
     const int v_sw = 4 * tj;                             // row % 4 == tj for every row this lane reads
 
-    // The tile loop is split in two levels so that NOTHING inside the hot inner loop touches the O
-    // accumulators except the MFMAs: when a row's maximum jumps (rare, see kRescaleLog2) the wave
-    // leaves the inner loop before using the tile, rescales in the cold outer block and re-enters
-    // at the same tile.  With the rescale written inside the hot loop the register allocator keeps
-    // a VGPR copy of all 128 accumulator registers and refreshes it on every iteration.
-    int t = t_begin;
-    bool resume = false;          // tile t was already awaited, announced and prefetched for
-    float m_pending = -INFINITY;
-    while (t < t_end) {
-    bool jumped = false;
-    for (; t < t_end; ++t) {
-        if (!resume) {
-            // tile t has landed once at most (tiles issued after it) * LD_PER_TILE loads are outstanding
-            const int ahead = (t_end - 1 - t) < (kStages - 2) ? (t_end - 1 - t) : (kStages - 2);
-            if (ahead >= 2) wait_vmcnt<2 * LD_PER_TILE>();
-            else if (ahead == 1) wait_vmcnt<LD_PER_TILE>();
-            else wait_vmcnt<0>();
-            __builtin_amdgcn_s_barrier();   // everyone's share of tile t is in LDS; everyone is done with tile t-1
-            if (t + kStages - 1 < t_end) issue_tile(t + kStages - 1);   // refills the stage tile t-1 used
-        }
-        resume = false;
+    auto stage_of = [&](int t) -> const unsigned char* { return smem + ((t - t_begin) % kStages) * L::STAGE; };
+    auto load_k = [&](const unsigned char* ks, int s) -> vec8 {
+        return *reinterpret_cast<const vec8*>(ks + k_rd + (((2 * s + h) ^ k_sw) * 16));
+    };
+    // V^T operand of PV step s: output block s % DB, key half s / DB.  The MFMA consumes accumulator
+    // registers 8*ksub .. 8*ksub+7 of S^T, i.e. keys 16*ksub + {4h..4h+3} and 16*ksub + 8 + {4h..4h+3}:
+    // two transposing reads of four keys each.
+    auto load_v = [&](const unsigned char* vs, int s) -> vec8 {
+        const int i = s % DB, ksub = s / DB;
+        const int off = v_rd + ((((4 * i + v_piece)) ^ v_sw) * 16);
+        const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4_t*)(vs + off + (16 * ksub) * L::ROWB));
+        const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4_t*)(vs + off + (16 * ksub + 8) * L::ROWB));
+        return __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+    constexpr int kAhead = 4;       // operand reads run this many MFMA steps ahead; sched_barrier pins the order
 
-        if (wave_active) {
-            const unsigned char* ks = smem + ((t - t_begin) % kStages) * L::STAGE;
-            const unsigned char* vs = ks + L::K_BYTES;
-
-            // ---- S^T = K Q^T for the tile's 32 keys ----
-            // Two accumulators: a dependent 32x32x16 MFMA waits out the full pipeline latency of its
-            // predecessor (~2.4 issue slots), so two interleaved chains roughly halve the Q K^T time
-            // (more chains cost more accumulator read-outs than they save).  Operand reads run
-            // kQkAhead k-steps ahead of the MFMAs; sched_barrier pins that order (left alone, the
-            // scheduler issues one whole chain after the other).
-            constexpr int kQkAhead = 8;
-            f32x16_t sacc, sacc1;
+    // S^T = K Q^T of one tile on its own (first tile only).  Two accumulators: a dependent 32x32x16
+    // MFMA waits out the pipeline latency of its predecessor, two interleaved chains hide half of it.
+    auto qk_tile = [&](int t, f32x16_t& sc) {
+        const unsigned char* ks = stage_of(t);
+        f32x16_t sc1;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) { sacc[v] = 0.f; sacc1[v] = 0.f; }
-            vec8 ka[KSTEPS];
+        for (int v = 0; v < 16; ++v) { sc[v] = 0.f; sc1[v] = 0.f; }
+        vec8 ka[KSTEPS];
 #pragma unroll
-            for (int s = 0; s < kQkAhead; ++s)
-                ka[s] = *reinterpret_cast<const vec8*>(ks + k_rd + (((2 * s + h) ^ k_sw) * 16));
+        for (int s = 0; s < kAhead; ++s) ka[s] = load_k(ks, s);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KSTEPS; s += 2) {
+            if (s + kAhead < KSTEPS) { ka[s + kAhead] = load_k(ks, s + kAhead); ka[s + kAhead + 1] = load_k(ks, s + kAhead + 1); }
+            sc = Tag::mfma(ka[s], qreg[s], sc);
+            sc1 = Tag::mfma(ka[s + 1], qreg[s + 1], sc1);
             __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
-            for (int s = 0; s < KSTEPS; s += 2) {
-                if (s + kQkAhead < KSTEPS) {
-                    ka[s + kQkAhead] = *reinterpret_cast<const vec8*>(ks + k_rd + (((2 * (s + kQkAhead) + h) ^ k_sw) * 16));
-                    ka[s + kQkAhead + 1] = *reinterpret_cast<const vec8*>(ks + k_rd + (((2 * (s + kQkAhead + 1) + h) ^ k_sw) * 16));
-                }
-                sacc = Tag::mfma(ka[s], qreg[s], sacc);
-                sacc1 = Tag::mfma(ka[s + 1], qreg[s + 1], sacc1);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-#pragma unroll
-            for (int v = 0; v < 16; ++v) sacc[v] += sacc1[v];
+        for (int v = 0; v < 16; ++v) sc[v] += sc1[v];
+    };
 
-            // ---- scale, causal mask, online softmax (log2 domain) ----
-            const int key0 = t * kBN;
-            const bool need_mask = (key0 + kBN) > (Nb - kM);
-            const int last_visible = Nb - kM + qi;     // row qi sees keys 0 .. Nb-16+qi
-            float mloc = -INFINITY;
+    vec8 pb[2];                     // P^T of the tile whose P V product comes next (two key halves)
+
+    // O^T += V^T P^T of tile t interleaved, MFMA by MFMA, with S^T = K Q^T of tile t+1: the single
+    // dependent Q K^T chain then advances every second issue slot, which is about its latency, and
+    // the eight independent O accumulators fill the slots in between.
+    auto pv_qk_tiles = [&](int t, f32x16_t& sc) {
+        const unsigned char* vs = stage_of(t) + L::K_BYTES;
+        const unsigned char* ks = stage_of(t + 1);
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                float x = sacc[v] * A.scale_log2;
-                if (need_mask) {
-                    const int key = key0 + 8 * (v >> 2) + 4 * h + (v & 3);
-                    x = key <= last_visible ? x : -INFINITY;
-                }
-                sacc[v] = x;
-                mloc = fmaxf(mloc, x);
+        for (int v = 0; v < 16; ++v) sc[v] = 0.f;
+        vec8 ka[KSTEPS], va[KSTEPS];
+#pragma unroll
+        for (int s = 0; s < kAhead; ++s) { va[s] = load_v(vs, s); ka[s] = load_k(ks, s); }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+            if (s + kAhead < KSTEPS) { va[s + kAhead] = load_v(vs, s + kAhead); ka[s + kAhead] = load_k(ks, s + kAhead); }
+            oacc[s % DB] = Tag::mfma(va[s], pb[s / DB], oacc[s % DB]);
+            sc = Tag::mfma(ka[s], qreg[s], sc);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto pv_tile = [&](int t) {     // last tile: nothing left to score
+        const unsigned char* vs = stage_of(t) + L::K_BYTES;
+        vec8 va[KSTEPS];
+#pragma unroll
+        for (int s = 0; s < kAhead; ++s) va[s] = load_v(vs, s);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+            if (s + kAhead < KSTEPS) va[s + kAhead] = load_v(vs, s + kAhead);
+            oacc[s % DB] = Tag::mfma(va[s], pb[s / DB], oacc[s % DB]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // Scale, causal mask and online softmax (log2 domain) of tile t's raw scores -> pb, m_run, l_run.
+    // Lazy rescale: the exponent reference m_run only moves when the tile's maximum exceeds it by
+    // more than kRescaleLog2 (P then stays below 2^kRescaleLog2, harmless in fp32/bf16).  If rows
+    // that already accumulated data need to move, nothing is changed and false is returned: the
+    // caller rescales the accumulators OUTSIDE the hot loop and calls again.  (With the rescale
+    // written inside the hot loop the register allocator keeps a VGPR copy of all 128 accumulator
+    // registers and refreshes it on every iteration.)
+    float m_pending = -INFINITY;
+    auto softmax_tile = [&](int t, const f32x16_t& sc) -> bool {
+        const int key0 = t * kBN;
+        const bool need_mask = (key0 + kBN) > (Nb - kM);
+        const int last_visible = Nb - kM + qi;     // row qi sees keys 0 .. Nb-16+qi
+        float x[16];
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            x[v] = sc[v] * A.scale_log2;
+            if (need_mask) {
+                const int key = key0 + 8 * (v >> 2) + 4 * h + (v & 3);
+                x[v] = key <= last_visible ? x[v] : -INFINITY;
             }
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-            // Lazy rescale: the exponent reference m_run only moves when the tile's maximum
-            // exceeds it by more than kRescaleLog2 (P then stays below 2^kRescaleLog2, harmless in
-            // fp32/bf16), so the 128 accumulator registers are rarely touched by the softmax.
-            const bool bump = mloc > m_run + kRescaleLog2;      // also true for the first finite maximum
-            if (__builtin_amdgcn_ballot_w64(bump && m_run != -INFINITY) != 0) {
-                m_pending = mloc;                               // accumulators hold data: rescale first
+            mloc = fmaxf(mloc, x[v]);
+        }
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+        const bool bump = mloc > m_run + kRescaleLog2;      // also true for the first finite maximum
+        if (__builtin_amdgcn_ballot_w64(bump && m_run != -INFINITY) != 0) {
+            m_pending = mloc;
+            return false;
+        }
+        const float m_new = bump ? mloc : m_run;            // a bump here starts from an empty row
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        m_run = m_new;
+        float psum = 0.f;
+        f32x8_t p0, p1;
+#pragma unroll
+        for (int v = 0; v < 8; ++v) {
+            p0[v] = fast_exp2(x[v] - m_safe);
+            p1[v] = fast_exp2(x[v + 8] - m_safe);
+            psum += p0[v] + p1[v];
+        }
+        l_run += psum;
+        pb[0] = Tag::pack(p0);
+        pb[1] = Tag::pack(p1);
+        return true;
+    };
+
+    // ---- first tile: scores and softmax; afterwards every iteration multiplies tile t by V while it
+    // scores tile t+1 ----
+    __builtin_amdgcn_s_barrier();                  // tile t_begin (awaited together with Q) is in LDS for all waves
+    f32x16_t sacc;
+    if (wave_active) {
+        qk_tile(t_begin, sacc);
+        softmax_tile(t_begin, sacc);               // rows are empty: cannot ask for a rescale
+    }
+    int t = t_begin;
+    const int t_last = t_end - 1;
+    bool redo = false;                             // the MFMA part of iteration t is done, only the softmax is repeated
+    while (t < t_last) {
+        bool jumped = false;
+        for (; t < t_last; ++t) {
+            if (!redo) {
+                // tile t+1 has landed once at most (tiles issued after it) * LD_PER_TILE loads are outstanding
+                const int later = (t_last - 1 - t) < (kStages - 3) ? (t_last - 1 - t) : (kStages - 3);
+                if (later >= 2) wait_vmcnt<2 * LD_PER_TILE>();
+                else if (later == 1) wait_vmcnt<LD_PER_TILE>();
+                else wait_vmcnt<0>();
+                __builtin_amdgcn_s_barrier();      // tile t+1 is in LDS for everyone; everyone is done with tile t-1
+                if (t + kStages - 1 < t_end) issue_tile(t + kStages - 1);   // refills the stage tile t-1 used
+                if (wave_active) pv_qk_tiles(t, sacc);
+            }
+            redo = false;
+            if (wave_active && !softmax_tile(t + 1, sacc)) {
                 jumped = true;
                 break;
             }
-            const float m_new = bump ? mloc : m_run;            // a bump here starts from an empty row
-            const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-            m_run = m_new;
-            float psum = 0.f;
+        }
+        if (jumped) {                              // cold: move the exponent reference of the rows that jumped
+            const bool bump = m_pending > m_run + kRescaleLog2;
+            const float alpha = (bump && m_run != -INFINITY) ? fast_exp2(m_run - m_pending) : 1.f;
+            if (bump) m_run = m_pending;
+            l_run *= alpha;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const float p = fast_exp2(sacc[v] - m_safe);
-                sacc[v] = p;
-                psum += p;
-            }
-            l_run += psum;
-
-            // ---- O^T += V^T P^T ----
-            // MFMA ksub feeds accumulator registers 8*ksub .. 8*ksub+7, i.e. keys
-            // 16*ksub + {4h..4h+3} and 16*ksub + 8 + {4h..4h+3}: two transposing reads.
+            for (int i = 0; i < DB; ++i)
 #pragma unroll
-            for (int ksub = 0; ksub < 2; ++ksub) {
-                f32x8_t pf;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) pf[e] = sacc[8 * ksub + e];
-                const vec8 pb = Tag::pack(pf);
-#pragma unroll
-                for (int i = 0; i < DB; ++i) {
-                    const int off = v_rd + ((((4 * i + v_piece)) ^ v_sw) * 16);
-                    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) s16x4_t*)(vs + off + (16 * ksub) * L::ROWB));
-                    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) s16x4_t*)(vs + off + (16 * ksub + 8) * L::ROWB));
-                    const s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                    oacc[i] = Tag::mfma(__builtin_bit_cast(vec8, both), pb, oacc[i]);
-                }
-            }
+                for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
+            redo = true;
         }
     }
-    if (jumped) {
-        const bool bump = m_pending > m_run + kRescaleLog2;
-        const float alpha = (bump && m_run != -INFINITY) ? fast_exp2(m_run - m_pending) : 1.f;
-        if (bump) m_run = m_pending;
-        l_run *= alpha;
-#pragma unroll
-        for (int i = 0; i < DB; ++i)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
-        resume = true;
-    }
-    }
+    if (wave_active) pv_tile(t_last);              // its scores were taken one iteration earlier
     __syncthreads();          // the tile buffers are free for the epilogue
 
     // ---- epilogue: partial statistics and O rows (through LDS for coalesced stores) ----
