@@ -399,6 +399,297 @@ __global__ __launch_bounds__(kThreads) void gated_delta_tape_kernel(GdnArgs A) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// Chunked form (fp32 state, one decay per head and step).
+//
+// The serial kernel above spends its time in T dependent steps that each need
+// two Dk-wide row reductions.  Unrolling the recurrence over a chunk of
+// C <= 16 steps moves every Dk-wide contraction out of the serial part:
+//
+//   G[s][t]  = g_{s+1} * ... * g_t                (products, never quotients: no underflow ratio)
+//   gam_t    = g_0 * ... * g_t
+//   S_t      = gam_t S_0 + sum_{s<=t} G[s][t] delta_s (x) k_s
+//   delta_t  = beta_t ( v_t - gam_t S_0 k_t - sum_{s<t} G[s][t] (k_s.k_t) delta_s )
+//   y_t      = gam_t S_0 q_t + sum_{s<=t} G[s][t] (k_s.q_t) delta_s
+//
+// so one fp32 MFMA product  [S_0 rows ; k rows] x [k | q]^T  gives S_0 k_t, S_0 q_t, k_s.k_t
+// and k_s.q_t at once, the step-to-step dependency shrinks to a 16x16 unit-triangular solve per
+// state row (a few registers per lane, no Dk-wide reduction), and the state update is one rank-C
+// MFMA product.  A masked or padded step is the identity step g = 1, beta = 0 (delta = 0) with
+// y forced to 0 (DFlashKernels.swift:150-197 leaves the state untouched and emits zeros).
+//
+// Workgroup: 16 state rows of one head (grid x = Dv/16, y = b*Hv + hv), 4 waves.
+// ---------------------------------------------------------------------------
+
+constexpr int kChunkRows = 16;
+constexpr int kChunkSteps = 16;
+
+template <int DK> struct GdnChunkLds {
+    static constexpr int LD = DK + 4;      // row pitch in floats: 16-byte pad spreads rows over the banks
+    float x[32][LD];                       // rows 0..15 state tile, rows 16..31 k_t
+    float y[32][LD];                       // rows 0..15 k_t, rows 16..31 q_t
+    float red[4][32][33];                  // per-wave partial products (each wave contracts Dk/4 channels)
+    float p[32][33];                       // [S_0 ; k] x [k | q]^T
+    float a[16][16];                       // a[s][t] = G[s][t] k_s.k_t for s < t, else 0
+    float c[16][16];                       // c[s][t] = G[s][t] k_s.q_t for s <= t, else 0
+    float dl[16][17];                      // delta_s of row r at dl[s][r]
+    float v[16][16];                       // v_t of row r at v[t][r]
+    float g[16], beta[16], gam[16], w[16]; // w[s] = G[s][15]: decay from step s to the end of the chunk
+    int on[16];
+};
+
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+typedef float f32x16v __attribute__((ext_vector_type(16)));
+
+template <int QUAD_LANE> __device__ __forceinline__ float quad_broadcast(float x) {
+    constexpr int ctrl = QUAD_LANE | (QUAD_LANE << 2) | (QUAD_LANE << 4) | (QUAD_LANE << 6);
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), ctrl, 0xf, 0xf, false));
+}
+
+// Steps S..15 of the unit-triangular solve for one state row held by a quad (lane q owns steps 4q..4q+3).
+template <int S> struct SolveStep {
+    static __device__ __forceinline__ void run(float (&acc)[4], const float4 (&arow)[16], const float (&bet)[16],
+                                               float (&dv)[16]) {
+        const float d = quad_broadcast<S / 4>(bet[S] * acc[S % 4]);
+        dv[S] = d;
+        acc[0] = fmaf(-arow[S].x, d, acc[0]);
+        acc[1] = fmaf(-arow[S].y, d, acc[1]);
+        acc[2] = fmaf(-arow[S].z, d, acc[2]);
+        acc[3] = fmaf(-arow[S].w, d, acc[3]);
+        if constexpr (S + 1 < 16) SolveStep<S + 1>::run(acc, arow, bet, dv);
+    }
+};
+
+template <bool HAS_MASK, int DK>
+__global__ __launch_bounds__(kThreads) void gated_delta_chunk_kernel(GdnArgs A) {
+    using Lds = GdnChunkLds<DK>;
+    extern __shared__ __align__(16) unsigned char gdn_chunk_smem[];
+    Lds& L = *reinterpret_cast<Lds*>(gdn_chunk_smem);
+    constexpr int E = DK / 64;             // channels per lane in the state-update product (16 lanes x E x 4 waves = DK)
+    static_assert(DK % 64 == 0, "chunked gated delta needs Dk to be a multiple of 64");
+
+    const int tid = threadIdx.x, lane = tid % 64, w = tid / 64;
+    const int bh = blockIdx.y;
+    const int b = bh / A.Hv, hv = bh % A.Hv;
+    const int hk = hv / (A.Hv / A.Hk);
+    const int row0 = blockIdx.x * kChunkRows;
+    const float* s_in = reinterpret_cast<const float*>(A.state_in) + ((size_t)bh * A.Dv + row0) * DK;
+    float* s_out = reinterpret_cast<float*>(A.state_out) + ((size_t)bh * A.Dv + row0) * DK;
+
+    constexpr int NV = kChunkRows * (DK / 4) / kThreads;      // float4 groups per thread of a 16 x DK tile
+    const int ts = tid / 16, tt = tid % 16;        // (s, t) for the tables, (t, r) for v / y / tape
+
+    if (A.T == 0) {                        // nothing to do but hand the state over
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int i = tid + u * kThreads, r = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
+            store4(s_out + (size_t)r * DK + c4, load4(s_in + (size_t)r * DK + c4));
+        }
+        return;
+    }
+
+    // Stage one chunk: every global load of the chunk (and of the state tile, first chunk only) is issued
+    // before the first conversion or LDS store, so the chunk pays one memory round trip, not one per array.
+    // Steps >= tc are identity steps.  Elem is the element type of q/k/v/g/beta.
+    auto stage = [&](auto elem_tag, int t0, int tc, bool with_state) {
+        using Elem = decltype(elem_tag);
+        const Elem* kp = reinterpret_cast<const Elem*>(A.k);
+        const Elem* qp = reinterpret_cast<const Elem*>(A.q);
+        const Elem* vp = reinterpret_cast<const Elem*>(A.v);
+        const Elem* gp = reinterpret_cast<const Elem*>(A.g);
+        const Elem* bp = reinterpret_cast<const Elem*>(A.beta);
+        float4 sv[NV], kv[NV], qv[NV];
+        const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (with_state) {
+#pragma unroll
+            for (int u = 0; u < NV; ++u) {
+                const int i = tid + u * kThreads, r = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
+                sv[u] = load4(s_in + (size_t)r * DK + c4);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int i = tid + u * kThreads, t = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
+            const int tl = t < tc ? t : tc - 1;           // clamped: always a valid address, selected away below
+            const size_t o = (((size_t)b * A.T + t0 + tl) * A.Hk + hk) * DK + c4;
+            kv[u] = load4(kp + o);
+            qv[u] = load4(qp + o);
+        }
+        const int tvl = ts < tc ? ts : tc - 1;
+        const float vv = to_float(vp[(((size_t)b * A.T + t0 + tvl) * A.Hv + hv) * A.Dv + row0 + tt]);
+        float gv = 1.f, bv = 0.f;
+        bool on = false;
+        if (tid < kChunkSteps) {
+            const int tl = tid < tc ? tid : tc - 1;
+            const size_t bt = (size_t)b * A.T + t0 + tl;
+            gv = to_float(gp[bt * A.Hv + hv]);
+            bv = to_float(bp[bt * A.Hv + hv]);
+            on = HAS_MASK ? mask_on(A.mask, A.mask_dtype, (int)bt) : true;
+            on = on && tid < tc;
+        }
+        if (with_state) {
+#pragma unroll
+            for (int u = 0; u < NV; ++u) {
+                const int i = tid + u * kThreads, r = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
+                store4(&L.x[r][c4], sv[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int i = tid + u * kThreads, t = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
+            const float4 k4 = t < tc ? kv[u] : zero4, q4 = t < tc ? qv[u] : zero4;
+            store4(&L.x[16 + t][c4], k4);
+            store4(&L.y[t][c4], k4);
+            store4(&L.y[16 + t][c4], q4);
+        }
+        L.v[ts][tt] = ts < tc ? vv : 0.f;
+        if (tid < kChunkSteps) {
+            L.on[tid] = on;
+            L.g[tid] = on ? gv : 1.f;
+            L.beta[tid] = on ? bv : 0.f;
+        }
+    };
+
+    for (int t0 = 0; t0 < A.T; t0 += kChunkSteps) {
+        const int tc = (A.T - t0) < kChunkSteps ? (A.T - t0) : kChunkSteps;
+        const bool last_chunk = t0 + kChunkSteps >= A.T;
+        if (A.in_dtype == DFLASH_BF16) stage(bf16_t{}, t0, tc, t0 == 0);
+        else if (A.in_dtype == DFLASH_F16) stage(f16_t{}, t0, tc, t0 == 0);
+        else stage(float{}, t0, tc, t0 == 0);
+        __syncthreads();
+
+        // ---- [S_0 ; k] x [k | q]^T, wave w contracting channels w*DK/4 .. +DK/4-1 ----
+        // A 32x32x2 fp32 MFMA takes lane l's a as row l%32, contraction index l/32 (b alike), so a float4
+        // per lane feeds four MFMAs whose index pairs are {e, 4+e} of an 8-channel group.
+        {
+            f32x16v acc;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+            const int kc0 = w * (DK / 4) + 4 * (lane / 32);
+#pragma unroll
+            for (int c = 0; c < DK / 32; ++c) {
+                const float4 a4 = *reinterpret_cast<const float4*>(&L.x[lane % 32][kc0 + 8 * c]);
+                const float4 b4 = *reinterpret_cast<const float4*>(&L.y[lane % 32][kc0 + 8 * c]);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.x, b4.x, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.y, b4.y, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.z, b4.z, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.w, b4.w, acc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) L.red[w][8 * (v / 4) + 4 * (lane / 32) + (v % 4)][lane % 32] = acc[v];
+        }
+        // decay products for the pair (s, t) = (ts, tt)
+        float G = 1.f;
+#pragma unroll
+        for (int j = 1; j < kChunkSteps; ++j) G *= (j > ts && j <= tt) ? L.g[j] : 1.f;
+        __syncthreads();
+        // sum the four partial products: the S_0 half (16 x 32) as two entries per thread, the k half
+        // straight into the coefficient tables of the pair (ts, tt)
+        {
+            auto red4 = [&](int r, int c) { return (L.red[0][r][c] + L.red[1][r][c]) + (L.red[2][r][c] + L.red[3][r][c]); };
+            L.p[ts][tt] = red4(ts, tt);
+            L.p[ts][16 + tt] = red4(ts, 16 + tt);
+            L.a[ts][tt] = ts < tt ? G * red4(16 + ts, tt) : 0.f;
+            L.c[ts][tt] = ts <= tt ? G * red4(16 + ts, 16 + tt) : 0.f;
+            if (ts == 0) L.gam[tt] = L.g[0] * G;
+            if (tt == kChunkSteps - 1) L.w[ts] = G;
+        }
+        __syncthreads();
+
+        // ---- unit-triangular solve for delta: wave 0, one quad per state row, lane q owns steps 4q..4q+3 ----
+        // The chain per step is multiply -> quad broadcast -> fused multiply-add; everything else (coefficients,
+        // betas, the LDS stores of delta) is kept off it.
+        if (w == 0) {
+            const int r = lane / 4, q = lane % 4;
+            float acc[4], bet[16], dv[16];
+            float4 arow[16];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] = fmaf(-L.gam[4 * q + e], L.p[r][4 * q + e], L.v[4 * q + e][r]);
+#pragma unroll
+            for (int s = 0; s < 16; ++s) {
+                arow[s] = *reinterpret_cast<const float4*>(&L.a[s][4 * q]);
+                bet[s] = L.beta[s];
+            }
+            SolveStep<0>::run(acc, arow, bet, dv);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float d = q == 0 ? dv[e] : q == 1 ? dv[4 + e] : q == 2 ? dv[8 + e] : dv[12 + e];
+                L.dl[4 * q + e][r] = d;
+            }
+        }
+        __syncthreads();
+
+        // ---- read-out and tape: thread (t, r) ----
+        {
+            const int t = ts, r = tt;
+            float yv = L.gam[t] * L.p[r][16 + t];
+#pragma unroll
+            for (int s = 0; s < kChunkSteps; ++s) yv = fmaf(L.c[s][t], L.dl[s][r], yv);
+            if (t < tc) {
+                const size_t o = (((size_t)b * A.T + t0 + t) * A.Hv + hv) * A.Dv + row0 + r;
+                store1_rt(A.y, A.in_dtype, o, L.on[t] ? yv : 0.f);
+                A.tape[o] = L.dl[t][r];
+            }
+        }
+
+        // ---- state: S <- gam_15 S_0 + sum_s w_s delta_s (x) k_s, as 16x16x4 fp32 MFMAs ----
+        // Lane l: a = row l%16, step 4*ks + l/16; b = column l%16 of the block; c = column l%16, rows 4*(l/16)+v.
+        // Column n of MFMA e stands for channel base + E*n + e, so a lane ends up with E consecutive channels.
+        {
+            const int n = lane % 16, kk = lane / 16;
+            const int base = w * 16 * E + E * n;
+            const float gam_end = L.gam[kChunkSteps - 1];
+            f32x4v cacc[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) cacc[e][v] = gam_end * L.x[4 * kk + v][base + e];
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const int s = 4 * ks + kk;
+                const float av = L.w[s] * L.dl[s][n];
+#pragma unroll
+                for (int e = 0; e < E; ++e)
+                    cacc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, L.y[s][base + e], cacc[e], 0, 0, 0);
+            }
+            if (last_chunk) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+#pragma unroll
+                    for (int e = 0; e < E; ++e) s_out[(size_t)(4 * kk + v) * DK + base + e] = cacc[e][v];
+            } else {
+                __syncthreads();           // every wave has read the old tile
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+#pragma unroll
+                    for (int e = 0; e < E; ++e) L.x[4 * kk + v][base + e] = cacc[e][v];
+                // the staging barrier of the next chunk orders these writes before their readers
+            }
+        }
+    }
+}
+
+template <int DK>
+static int launch_gdn_chunk(hipStream_t st, const GdnArgs& A, int B) {
+    static bool attr_done_dev[64][2];      // the attribute is per device and per instantiation
+    const size_t lds = sizeof(GdnChunkLds<DK>);
+    const int mi = A.mask ? 1 : 0;
+    int dev = 0;
+    DFLASH_HIP_TRY(hipGetDevice(&dev));
+    bool* attr_done = attr_done_dev[dev & 63];
+    if (!attr_done[mi]) {
+        if (mi) DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<true, DK>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        else DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<false, DK>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_done[mi] = true;
+    }
+    dim3 grid(A.Dv / kChunkRows, B * A.Hv);
+    LaunchBracket br(DFLASH_KERNEL_GDN_FORWARD, st);
+    if (A.mask) hipLaunchKernelGGL((gated_delta_chunk_kernel<true, DK>), grid, dim3(kThreads), lds, st, A);
+    else hipLaunchKernelGGL((gated_delta_chunk_kernel<false, DK>), grid, dim3(kThreads), lds, st, A);
+    DFLASH_HIP_TRY(hipGetLastError());
+    return DFLASH_OK;
+}
+
 template <typename StateT>
 static int launch_gdn_state(hipStream_t st, const GdnArgs& A, int B, int g_ndim, int Dk) {
     const bool vec = g_ndim == 4;
@@ -472,6 +763,12 @@ extern "C" int dflash_gated_delta_tape(void* stream, const void* q, const void* 
     A.q = q; A.k = k; A.v = v; A.g = g; A.beta = beta; A.mask = mask;
     A.state_in = state_in; A.state_out = state_out; A.y = y; A.tape = tape_out;
     A.in_dtype = in_dtype; A.mask_dtype = mask_dtype; A.T = T; A.Hk = Hk; A.Hv = Hv; A.Dv = Dv;
+    if (state_dtype == DFLASH_F32 && g_ndim == 3 && Dv % kChunkRows == 0 && T > 0) {
+        // fp32 state with one decay per head and step: chunked form
+        if (Dk == 64) return launch_gdn_chunk<64>((hipStream_t)stream, A, B);
+        if (Dk == 128) return launch_gdn_chunk<128>((hipStream_t)stream, A, B);
+        if (Dk == 256) return launch_gdn_chunk<256>((hipStream_t)stream, A, B);
+    }
     switch (state_dtype) {
         case DFLASH_F32: return launch_gdn_state<float>((hipStream_t)stream, A, B, g_ndim, Dk);
         case DFLASH_BF16: return launch_gdn_state<bf16_t>((hipStream_t)stream, A, B, g_ndim, Dk);
