@@ -149,6 +149,21 @@ int dflash_sdpa_block_causal(void* stream,
                              const int32_t* kv_len_dev,
                              void* workspace, size_t workspace_bytes);
 
+/* The same attention with the reference's optional additive mask (masked partials
+ * kernel, DFlashKernels.swift:546-555; selected at :783-787).  mask [B, Hq, M, N]
+ * contiguous, in `dtype` (the reference casts it to the input type, :784).  A key
+ * is used when it passes the block-causal rule AND its mask value is at least the
+ * lowest finite value of `dtype` (:551); the mask value is added to the scaled
+ * score (:553).  A row without any usable key gets zeros (:711) and lse = -inf.
+ * ---------------------------------------------------------------------- */
+int dflash_sdpa_block_causal_masked(void* stream,
+                                    const void* q, const void* k, const void* v, const void* mask,
+                                    void* out, float* lse, int dtype, float scale,
+                                    int B, int Hq, int Hk, int M, int N, int D,
+                                    int64_t kv_batch_stride, int64_t kv_head_stride,
+                                    const int32_t* kv_len_dev,
+                                    void* workspace, size_t workspace_bytes);
+
 /* The same attention with the block's K/V append fused in: the verify forward's
  * KVCacheSimple.update (mlx-swift-lm, reached from the attention layer the
  * reference's batchedSDPA2Pass was written for) followed by the SDPA, in one launch

@@ -333,7 +333,8 @@ def sdpa_block_causal(q, k, v, scale, mask=None, *, dtype=np.float64):
     Q [B,Hq,M,D]; K,V [B,Hk,N,D] where N already includes the M block tokens;
     row i sees keys ``0 .. N-M+i`` (DFlashKernels.swift:614).  GQA head mapping
     ``hk = hq // (Hq/Hk)`` (:575).  ``mask`` is an optional additive
-    [B,Hq,M,N] (:548-553).  Returns (O [B,Hq,M,D], lse [B,Hq,M]) in ``dtype``;
+    [B,Hq,M,N] (:548-553); -inf entries drop the key, a row left without keys
+    yields zeros (:711).  Returns (O [B,Hq,M,D], lse [B,Hq,M]) in ``dtype``;
     ``lse = max + log(sum exp)`` of the scaled, masked scores (natural log).
 
     This is what ``sdpaFallback`` (:818-828) asks of
@@ -355,13 +356,18 @@ def sdpa_block_causal(q, k, v, scale, mask=None, *, dtype=np.float64):
             hk = h // rf
             s = (q[b, h] * dtype(scale)) @ k[b, hk].T          # scale folded into Q (:594)
             if mask is not None:
-                s = s + np.asarray(mask[b, h], dtype=dtype)
+                mk = np.asarray(mask[b, h], dtype=dtype)
+                # a key is used only when its mask value is a finite number of the input type (:551);
+                # the mask value is added to the score (:553)
+                s = np.where(mk > -np.inf, s + mk, -np.inf)
             s = np.where(visible, s, -np.inf)
             m = s.max(axis=-1, keepdims=True)
-            p = np.exp(s - m)
+            m_safe = np.where(np.isfinite(m), m, 0.0)
+            p = np.exp(s - m_safe)
             l = p.sum(axis=-1, keepdims=True)
-            out[b, h] = (p @ v[b, hk]) / l
-            lse[b, h] = (m + np.log(l))[:, 0]
+            with np.errstate(divide="ignore", invalid="ignore"):
+                out[b, h] = np.where(l > 0, (p @ v[b, hk]) / np.where(l > 0, l, 1.0), 0.0)   # no usable key: zeros (:711)
+                lse[b, h] = np.where(l > 0, m_safe + np.log(l), -np.inf)[:, 0]
     return out, lse
 
 

@@ -32,6 +32,7 @@ SIGNATURES = {
     "dflash_gated_delta_tape": (i32, [vp, vp, vp, vp, vp, i32, vp, i32, vp, vp, i32, vp, vp, vp, i32] + [i32] * 6),
     "dflash_sdpa_workspace_bytes": (sz, [i32] * 6),
     "dflash_sdpa_block_causal": (i32, [vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp, vp, sz]),
+    "dflash_sdpa_block_causal_masked": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp, vp, sz]),
     "dflash_sdpa_block_causal_append": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp, vp, sz]),
     "dflash_match_acceptance_length": (i32, [vp, vp, vp, i32, vp]),
     "dflash_accept_commit": (i32, [vp, vp, vp, i32, vp, vp]),

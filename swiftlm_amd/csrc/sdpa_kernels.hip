@@ -80,6 +80,7 @@ struct SdpaArgs {
     float* part_m;   // [B*Hq*16, S]   running max, log2 units
     float* part_l;   // [B*Hq*16, S]   sum of exp2
     const int32_t* kv_len_dev;
+    const uint16_t* mask;    // additive mask [B,Hq,16,N] in the input type (DFlashKernels.swift:548-553), or null
     int64_t kv_batch_stride, kv_head_stride;
     float scale_log2;   // scale * log2(e)
     int Hq, Hk, G, N, S, groups_per_kv;
@@ -154,7 +155,11 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 // 4*j + q supplies the address of 4 channels of key row j; lane i receives channel
 // (i % 4) of the address given by lane 4*r + i/4 as its r-th element, i.e. four
 // consecutive keys of channel d0 + i when lane 4*j + q points at V[k0 + j][d0 + 4q].
-template <typename Tag, int D>
+// MASKED adds the reference's optional additive mask: a key is used when it passes the causal rule
+// and its mask value is at least the lowest finite value of the input type, and the mask value is
+// added to the scaled score (DFlashKernels.swift:550-553, :614-623).  The mask is read with plain
+// loads inside the softmax; that instantiation is for signature parity, not for speed.
+template <typename Tag, int D, bool MASKED>
 __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs A) {
     typedef typename Tag::vec8 vec8;
     typedef SdpaLds<D> L;
@@ -394,9 +399,24 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
         const int last_visible = Nb - kM + qi;     // row qi sees keys 0 .. Nb-16+qi
         float x[16];
         float mloc = -INFINITY;
+        float mk[16];
+        if constexpr (MASKED) {
+            const uint16_t* mrow = A.mask + row_id * (size_t)A.N;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                int key = key0 + 8 * (v >> 2) + 4 * h + (v & 3);
+                key = key < A.N ? key : A.N - 1;               // keys past the end fail the causal rule anyway
+                mk[v] = row_valid ? Tag::to_f32(mrow[key]) : 0.f;
+            }
+        }
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             x[v] = sc[v] * A.scale_log2;
+            if constexpr (MASKED) {
+                // -inf (or NaN) drops the key; a finite mask value, however low, keeps it in the softmax
+                x[v] = mk[v] >= -3.4028234663852886e38f ? fmaxf(fmaf(mk[v], 1.4426950408889634f, x[v]), -3.4028234663852886e38f)
+                                                         : -INFINITY;
+            }
             if (need_mask) {
                 const int key = key0 + 8 * (v >> 2) + 4 * h + (v & 3);
                 x[v] = key <= last_visible ? x[v] : -INFINITY;
@@ -616,11 +636,11 @@ static size_t ws_layout(int B, int Hq, int S, int D, size_t* off_m, size_t* off_
     return (o + 255) & ~(size_t)255;
 }
 
-template <typename Tag, int D>
+template <typename Tag, int D, bool MASKED>
 static int launch_sdpa(hipStream_t st, const SdpaArgs& A, const CombineArgs& C, int B) {
     typedef SdpaLds<D> L;
     static_assert(L::BYTES <= 160 * 1024, "tile buffers must fit the 160 KB LDS of a gfx950 CU");
-    auto kern = sdpa_partial_kernel<Tag, D>;
+    auto kern = sdpa_partial_kernel<Tag, D, MASKED>;
     // Raise the dynamic LDS limit above the 64 KB default, once per process.
     static const hipError_t attr_rc =
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::BYTES);
@@ -653,7 +673,7 @@ extern "C" size_t dflash_sdpa_workspace_bytes(int B, int Hq, int Hk, int M, int 
 }
 
 static int sdpa_common(void* stream, const void* q, const void* k, const void* v, const void* k_new, const void* v_new,
-                       void* k_cache, void* v_cache, void* out, float* lse, int dtype, float scale, int B, int Hq, int Hk,
+                       void* k_cache, void* v_cache, const void* mask, void* out, float* lse, int dtype, float scale, int B, int Hq, int Hk,
                        int M, int N, int D, int64_t kv_batch_stride, int64_t kv_head_stride, const int32_t* kv_len_dev,
                        void* workspace, size_t workspace_bytes) {
     int rc = ensure_init();
@@ -690,6 +710,7 @@ static int sdpa_common(void* stream, const void* q, const void* k, const void* v
     A.part_m = (float*)((char*)workspace + om);
     A.part_l = (float*)((char*)workspace + ol);
     A.kv_len_dev = kv_len_dev;
+    A.mask = (const uint16_t*)mask;
     A.kv_batch_stride = kv_batch_stride; A.kv_head_stride = kv_head_stride;
     A.scale_log2 = scale * 1.4426950408889634f;
     A.Hq = Hq; A.Hk = Hk; A.G = G; A.N = N; A.S = S; A.groups_per_kv = groups; A.rows_total = B * Hq * kM;
@@ -699,15 +720,19 @@ static int sdpa_common(void* stream, const void* q, const void* k, const void* v
     C.out = (uint16_t*)out; C.lse = lse; C.S = S;
 
     hipStream_t st = (hipStream_t)stream;
-    if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa<Bf16Tag, 256>(st, A, C, B) : launch_sdpa<Bf16Tag, 128>(st, A, C, B);
-    return D == 256 ? launch_sdpa<F16Tag, 256>(st, A, C, B) : launch_sdpa<F16Tag, 128>(st, A, C, B);
+    if (mask) {
+        if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa<Bf16Tag, 256, true>(st, A, C, B) : launch_sdpa<Bf16Tag, 128, true>(st, A, C, B);
+        return D == 256 ? launch_sdpa<F16Tag, 256, true>(st, A, C, B) : launch_sdpa<F16Tag, 128, true>(st, A, C, B);
+    }
+    if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa<Bf16Tag, 256, false>(st, A, C, B) : launch_sdpa<Bf16Tag, 128, false>(st, A, C, B);
+    return D == 256 ? launch_sdpa<F16Tag, 256, false>(st, A, C, B) : launch_sdpa<F16Tag, 128, false>(st, A, C, B);
 }
 
 extern "C" int dflash_sdpa_block_causal(void* stream, const void* q, const void* k, const void* v, void* out,
                                         float* lse, int dtype, float scale, int B, int Hq, int Hk, int M, int N,
                                         int D, int64_t kv_batch_stride, int64_t kv_head_stride,
                                         const int32_t* kv_len_dev, void* workspace, size_t workspace_bytes) {
-    return sdpa_common(stream, q, k, v, nullptr, nullptr, nullptr, nullptr, out, lse, dtype, scale, B, Hq, Hk, M, N, D,
+    return sdpa_common(stream, q, k, v, nullptr, nullptr, nullptr, nullptr, nullptr, out, lse, dtype, scale, B, Hq, Hk, M, N, D,
                        kv_batch_stride, kv_head_stride, kv_len_dev, workspace, workspace_bytes);
 }
 
@@ -717,6 +742,16 @@ extern "C" int dflash_sdpa_block_causal_append(void* stream, const void* q, void
                                                int64_t kv_batch_stride, int64_t kv_head_stride,
                                                const int32_t* cache_len_dev, void* workspace, size_t workspace_bytes) {
     DFLASH_REQUIRE(k_new && v_new && k_cache && v_cache, "sdpa (append): null pointer");
-    return sdpa_common(stream, q, k_cache, v_cache, k_new, v_new, k_cache, v_cache, out, lse, dtype, scale, B, Hq, Hk, M,
+    return sdpa_common(stream, q, k_cache, v_cache, k_new, v_new, k_cache, v_cache, nullptr, out, lse, dtype, scale, B, Hq, Hk, M,
                        N, D, kv_batch_stride, kv_head_stride, cache_len_dev, workspace, workspace_bytes);
+}
+
+extern "C" int dflash_sdpa_block_causal_masked(void* stream, const void* q, const void* k, const void* v,
+                                               const void* mask, void* out, float* lse, int dtype, float scale, int B,
+                                               int Hq, int Hk, int M, int N, int D, int64_t kv_batch_stride,
+                                               int64_t kv_head_stride, const int32_t* kv_len_dev, void* workspace,
+                                               size_t workspace_bytes) {
+    DFLASH_REQUIRE(mask, "sdpa (masked): null mask");
+    return sdpa_common(stream, q, k, v, nullptr, nullptr, nullptr, nullptr, mask, out, lse, dtype, scale, B, Hq, Hk, M, N, D,
+                       kv_batch_stride, kv_head_stride, kv_len_dev, workspace, workspace_bytes);
 }

@@ -143,17 +143,22 @@ class DFlashKernels:
 
         queries [B,Hq,16,D]; keys/values [B,Hk,N,D] with N including the 16 block
         tokens (a view into a larger cache is fine as long as the last dimension is
-        contiguous and rows are D apart).  Returns None where the reference returns
-        nil (unsupported shape/dtype).  ``return_lse`` additionally returns the
+        contiguous and rows are D apart).  ``mask`` is the reference's optional additive
+        mask [B,Hq,16,N].  Returns None where the reference returns nil (unsupported
+        shape/dtype).  ``return_lse`` additionally returns the
         float32 logsumexp [B,Hq,16]; ``kv_len`` (int32 [B] on the device) gives
         per-sequence key counts for ragged batches."""
         if queries.dim() != 4 or keys.dim() != 4 or values.dim() != 4:
             return None
-        if mask is not None:
-            return None   # additive masks are not covered by the HIP kernel
-        _dev(queries, keys, values, kv_len, workspace)
+        _dev(queries, keys, values, kv_len, workspace, mask)
         B, Hq, M, D = queries.shape
         Hk, N = keys.shape[1], keys.shape[2]
+        if mask is not None:
+            # additive [B,Hq,16,N] (anything that broadcasts to it), cast to the input type (:783-787)
+            try:
+                mask = mask.to(queries.dtype).expand(B, Hq, M, N).contiguous()
+            except RuntimeError:
+                raise DFlashError(f"batched_sdpa_2pass: mask {tuple(mask.shape)} does not broadcast to {(B, Hq, M, N)}")
         if values.shape != keys.shape or values.shape[3] != D or keys.dtype != queries.dtype or values.dtype != queries.dtype:
             return None
         queries = queries.contiguous()
@@ -171,10 +176,13 @@ class DFlashKernels:
             code = _code(queries)
         except DFlashUnsupported:
             return None
-        rc = lib.dflash_sdpa_block_causal(
-            _stream(), _ptr(queries), _ptr(keys), _ptr(values), _ptr(out), _ptr(lse), code, float(scale),
-            B, Hq, Hk, M, N, D, keys.stride(0), keys.stride(1), _ptr(kv_len), _ptr(workspace),
-            workspace.numel() * workspace.element_size())
+        tail = (code, float(scale), B, Hq, Hk, M, N, D, keys.stride(0), keys.stride(1), _ptr(kv_len), _ptr(workspace),
+                workspace.numel() * workspace.element_size())
+        if mask is None:
+            rc = lib.dflash_sdpa_block_causal(_stream(), _ptr(queries), _ptr(keys), _ptr(values), _ptr(out), _ptr(lse), *tail)
+        else:
+            rc = lib.dflash_sdpa_block_causal_masked(_stream(), _ptr(queries), _ptr(keys), _ptr(values), _ptr(mask),
+                                                     _ptr(out), _ptr(lse), *tail)
         if rc == _lib.UNSUPPORTED:
             return None
         _lib.check(rc, "batched_sdpa_2pass")

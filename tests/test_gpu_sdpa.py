@@ -142,6 +142,47 @@ def test_sdpa_ragged_batch(gpu_lib):
         np.testing.assert_allclose(host(single), host(out[b:b + 1]), rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("cfg", [(1, 16, 2, 100, 256), (2, 4, 2, 333, 128), (1, 16, 2, 1003, 256)],
+                         ids=["L100_D256", "B2_L333_D128", "L1003_odd_row_pitch"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_sdpa_additive_mask_matches_oracle(gpu_lib, cfg, dtype):
+    """The masked partials kernel (DFlashKernels.swift:546-555): finite biases, dropped keys
+    (-inf), a value at the lowest finite number of the type (still a usable key, :551), and one
+    row with no usable key at all (zeros, :711)."""
+    from swiftlm_amd import DFlashKernels as K
+
+    B, Hq, Hk, L, D = cfg
+    N = L + 16
+    q, k, v = gpu_inputs(B * 77 + L, B, Hq, Hk, L, D, dtype)
+    g = torch.Generator(device="cuda").manual_seed(L)
+    mask = torch.randn(B, Hq, 16, N, generator=g, device="cuda")
+    drop = torch.rand(B, Hq, 16, N, generator=g, device="cuda") < 0.3
+    mask = mask.masked_fill(drop, float("-inf"))
+    mask[0, 0, 5, :] = float("-inf")                      # no usable key
+    mask[0, 1, 2, :] = float("-inf")
+    mask[0, 1, 2, 3] = torch.finfo(dtype).min             # only key 3, at the lowest finite value
+    mask = mask.to(dtype)
+    scale = 1.0 / math.sqrt(D)
+    out, lse = K.batched_sdpa_2pass(q, k, v, scale, mask, return_lse=True)
+    torch.cuda.synchronize()
+    ow, lw = O.sdpa_block_causal(host(q), host(k), host(v), scale, host(mask).astype(np.float64))
+    np.testing.assert_allclose(host(out), ow, **OUT_TOL)
+    got_lse = host(lse)
+    assert np.all(got_lse[0, 0, 5] == -np.inf) and np.all(host(out)[0, 0, 5] == 0)
+    np.testing.assert_allclose(host(out)[0, 1, 2], host(v)[0, 0, 3], **OUT_TOL)      # all weight on key 3
+    fin = np.isfinite(lw) & (np.abs(lw) < 1e30)
+    np.testing.assert_allclose(got_lse[fin], lw[fin], **LSE_TOL)
+
+
+def test_sdpa_broadcast_mask_and_zero_mask(gpu_lib):
+    from swiftlm_amd import DFlashKernels as K
+
+    q, k, v = gpu_inputs(11, 1, 16, 2, 200, 256)
+    plain = K.batched_sdpa_2pass(q, k, v, 1.0 / 16)
+    zero = K.batched_sdpa_2pass(q, k, v, 1.0 / 16, torch.zeros(1, 1, 16, 216, device="cuda"))
+    assert torch.equal(plain, zero)
+
+
 def test_sdpa_unsupported_shapes_return_none(gpu_lib):
     """The reference's guards (DFlashKernels.swift:744-758): nil instead of an error."""
     from swiftlm_amd import DFlashKernels as K, DFlashUnsupported

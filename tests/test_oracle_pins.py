@@ -388,6 +388,26 @@ def test_sdpa_additive_mask():
     np.testing.assert_allclose(o, ow, rtol=1e-12)
 
 
+def test_sdpa_additive_mask_bias_and_empty_rows():
+    """A finite mask is a bias on the score (DFlashKernels.swift:553): adding log(w_n) weights key n
+    by w_n in the softmax.  A row whose keys are all dropped yields zeros, not NaN (:711)."""
+    q, k, v = (a.astype(np.float64) for a in O.make_sdpa_inputs(6, B=1, Hq=2, Hk=1, M=16, L=8, D=8))
+    N = 24
+    rng = np.random.default_rng(0)
+    w = rng.uniform(0.5, 2.0, size=(1, 2, 16, N))
+    o, lse = O.sdpa_block_causal(q, k, v, 0.3, np.log(w))
+    s = np.einsum("bhmd,bhnd->bhmn", q * 0.3, np.repeat(k, 2, axis=1))
+    vis = np.arange(N)[None, :] <= (N - 16 + np.arange(16))[:, None]
+    p = np.where(vis, w * np.exp(s), 0.0)
+    np.testing.assert_allclose(o, np.einsum("bhmn,bhnd->bhmd", p / p.sum(-1, keepdims=True), np.repeat(v, 2, axis=1)), rtol=1e-12)
+    np.testing.assert_allclose(lse, np.log(p.sum(-1)), rtol=1e-12)
+    mask = np.zeros((1, 2, 16, N))
+    mask[0, 1, 3, :] = -np.inf
+    o, lse = O.sdpa_block_causal(q, k, v, 0.3, mask)
+    assert np.all(o[0, 1, 3] == 0.0) and lse[0, 1, 3] == -np.inf
+    assert np.isfinite(o).all()
+
+
 @pytest.mark.parametrize("blocks", [32, 64])
 def test_sdpa_2pass_agrees_with_single_pass(blocks):
     q, k, v = O.make_sdpa_inputs(5, B=1, Hq=4, Hk=2, M=16, L=200, D=16)
