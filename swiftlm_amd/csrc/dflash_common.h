@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
@@ -45,13 +46,18 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 int ensure_init();           // per-device one-time setup; 0 or negative hip error
 int num_compute_units();     // of the current device (cached)
 
-// Brackets one kernel launch with the caller's events when the thread was armed by
-// dflash_profile_next_launch(); otherwise does nothing.
+// Launches one kernel.  When the thread was armed by dflash_profile_next_launch() for this kernel id,
+// the caller's events are attached to the dispatch itself (hipExtLaunchKernelGGL), so their elapsed
+// time is the kernel's own begin-to-end duration, as a profiler reports it, not a bracket around it.
 struct LaunchBracket {
     hipStream_t stream;
-    hipEvent_t stop;
+    hipEvent_t start, stop;
     LaunchBracket(int kernel_id, hipStream_t st);
-    ~LaunchBracket() { if (stop) (void)hipEventRecord(stop, stream); }
+    template <typename K, typename... Args>
+    void launch(K kern, dim3 grid, dim3 block, size_t lds, Args... args) {
+        if (start) hipExtLaunchKernelGGL(kern, grid, block, lds, stream, start, stop, 0, args...);
+        else hipLaunchKernelGGL(kern, grid, block, lds, stream, args...);
+    }
     LaunchBracket(const LaunchBracket&) = delete;
     LaunchBracket& operator=(const LaunchBracket&) = delete;
 };

@@ -52,10 +52,9 @@ int num_compute_units() {
 struct ArmedBracket { hipEvent_t start = nullptr, stop = nullptr; };
 static thread_local ArmedBracket g_bracket[DFLASH_KERNEL_COUNT];
 
-LaunchBracket::LaunchBracket(int kernel_id, hipStream_t st) : stream(st), stop(nullptr) {
+LaunchBracket::LaunchBracket(int kernel_id, hipStream_t st) : stream(st), start(nullptr), stop(nullptr) {
     ArmedBracket& a = g_bracket[kernel_id];
-    if (!a.start) return;
-    (void)hipEventRecord(a.start, st);
+    start = a.start;
     stop = a.stop;
     a.start = a.stop = nullptr;
 }

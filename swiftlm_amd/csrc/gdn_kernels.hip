@@ -159,10 +159,10 @@ static int launch_replay_nr(hipStream_t st, const ReplayBatch& P, const ReplayAr
     LaunchBracket br(DFLASH_KERNEL_TAPE_REPLAY, st);
     if (wg1 >= 16L * cus && A.Dv >= RPP * 4) {
         dim3 grid((A.Dv + RPP * 4 - 1) / (RPP * 4), B * A.Hv, n_layers);
-        hipLaunchKernelGGL((tape_replay_kernel<StateT, VEC_G, DK, 4>), grid, dim3(kThreads), 0, st, P, A);
+        br.launch(tape_replay_kernel<StateT, VEC_G, DK, 4>, grid, dim3(kThreads), 0, P, A);
     } else {
         dim3 grid((A.Dv + RPP - 1) / RPP, B * A.Hv, n_layers);
-        hipLaunchKernelGGL((tape_replay_kernel<StateT, VEC_G, DK, 1>), grid, dim3(kThreads), 0, st, P, A);
+        br.launch(tape_replay_kernel<StateT, VEC_G, DK, 1>, grid, dim3(kThreads), 0, P, A);
     }
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
@@ -684,8 +684,8 @@ static int launch_gdn_chunk(hipStream_t st, const GdnArgs& A, int B) {
     }
     dim3 grid(A.Dv / kChunkRows, B * A.Hv);
     LaunchBracket br(DFLASH_KERNEL_GDN_FORWARD, st);
-    if (A.mask) hipLaunchKernelGGL((gated_delta_chunk_kernel<true, DK>), grid, dim3(kThreads), lds, st, A);
-    else hipLaunchKernelGGL((gated_delta_chunk_kernel<false, DK>), grid, dim3(kThreads), lds, st, A);
+    if (A.mask) br.launch(gated_delta_chunk_kernel<true, DK>, grid, dim3(kThreads), lds, A);
+    else br.launch(gated_delta_chunk_kernel<false, DK>, grid, dim3(kThreads), lds, A);
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
 }
@@ -697,10 +697,10 @@ static int launch_gdn_state(hipStream_t st, const GdnArgs& A, int B, int g_ndim,
     case DKV: {                                                                                        \
         dim3 grid((A.Dv + (kThreads / LPRV) - 1) / (kThreads / LPRV), B * A.Hv);                       \
         LaunchBracket br(DFLASH_KERNEL_GDN_FORWARD, st);                                               \
-        if (vec && A.mask) hipLaunchKernelGGL((gated_delta_tape_kernel<StateT, true, true, DKV, LPRV>), grid, dim3(kThreads), 0, st, A);        \
-        else if (vec) hipLaunchKernelGGL((gated_delta_tape_kernel<StateT, true, false, DKV, LPRV>), grid, dim3(kThreads), 0, st, A);            \
-        else if (A.mask) hipLaunchKernelGGL((gated_delta_tape_kernel<StateT, false, true, DKV, LPRV>), grid, dim3(kThreads), 0, st, A);         \
-        else hipLaunchKernelGGL((gated_delta_tape_kernel<StateT, false, false, DKV, LPRV>), grid, dim3(kThreads), 0, st, A);                    \
+        if (vec && A.mask) br.launch(gated_delta_tape_kernel<StateT, true, true, DKV, LPRV>, grid, dim3(kThreads), 0, A);        \
+        else if (vec) br.launch(gated_delta_tape_kernel<StateT, true, false, DKV, LPRV>, grid, dim3(kThreads), 0, A);            \
+        else if (A.mask) br.launch(gated_delta_tape_kernel<StateT, false, true, DKV, LPRV>, grid, dim3(kThreads), 0, A);         \
+        else br.launch(gated_delta_tape_kernel<StateT, false, false, DKV, LPRV>, grid, dim3(kThreads), 0, A);                    \
         DFLASH_HIP_TRY(hipGetLastError());                                                             \
         return DFLASH_OK;                                                                              \
     }

@@ -648,12 +648,12 @@ static int launch_sdpa(hipStream_t st, const SdpaArgs& A, const CombineArgs& C, 
     dim3 grid(A.S, A.Hk * A.groups_per_kv, B);
     {
         LaunchBracket br(DFLASH_KERNEL_SDPA_PARTIAL, st);
-        hipLaunchKernelGGL(kern, grid, dim3(kSdpaThreads), L::BYTES, st, A);
+        br.launch(kern, grid, dim3(kSdpaThreads), L::BYTES, A);
     }
     DFLASH_HIP_TRY(hipGetLastError());
     {
         LaunchBracket br(DFLASH_KERNEL_SDPA_COMBINE, st);
-        hipLaunchKernelGGL((sdpa_combine_kernel<Tag, D>), dim3(B * A.Hq * kM), dim3(kSdpaThreads), 0, st, C);
+        br.launch(sdpa_combine_kernel<Tag, D>, dim3(B * A.Hq * kM), dim3(kSdpaThreads), 0, C);
     }
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
