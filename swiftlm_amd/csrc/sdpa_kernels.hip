@@ -36,7 +36,11 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(8))) float f32x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;   // one 16-byte global/LDS access
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
 
 constexpr int kSdpaThreads = 256;
 constexpr int kBN = 32;             // keys per tile
@@ -52,6 +56,7 @@ struct Bf16Tag {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
     static __device__ __forceinline__ vec8 pack(f32x8_t x) { return __builtin_convertvector(x, vec8); }
+    static __device__ __forceinline__ bf16x4_t pack4(f32x4_t x) { return __builtin_convertvector(x, bf16x4_t); }
     static __device__ __forceinline__ uint16_t cvt(float x) { return f32_to_bf16_bits(x); }
     static __device__ __forceinline__ float to_f32(uint16_t x) { return __uint_as_float(((uint32_t)x) << 16); }
 };
@@ -61,6 +66,7 @@ struct F16Tag {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
     static __device__ __forceinline__ vec8 pack(f32x8_t x) { return __builtin_convertvector(x, vec8); }
+    static __device__ __forceinline__ f16x4_t pack4(f32x4_t x) { return __builtin_convertvector(x, f16x4_t); }
     static __device__ __forceinline__ uint16_t cvt(float x) {
         _Float16 hf = (_Float16)x;
         return *reinterpret_cast<uint16_t*>(&hf);
@@ -99,8 +105,8 @@ template <int D> struct SdpaLds {
     static constexpr int K_BYTES = kBN * ROWB;
     static constexpr int STAGE = 2 * K_BYTES;
     static constexpr int LPW = (kBN / RPI) / 4;      // load instructions per wave per tile and operand
-    static constexpr int OS = D + 4;                 // epilogue O row stride, floats
-    static constexpr int EPI = 4 * 32 * OS * 4;
+    static constexpr int EROW = D * 2 + 16;          // epilogue O row pitch, bytes
+    static constexpr int EPI = 4 * 32 * EROW;
     static constexpr int BYTES = kStages * STAGE > EPI ? kStages * STAGE : EPI;
 };
 
@@ -498,32 +504,35 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
         A.part_l[row_id * A.S + split] = l_tot;
     }
     if (wave_active) {
-        float* os = reinterpret_cast<float*>(smem) + wave * 32 * L::OS;
+        // Rows are rounded to the input type first and staged as such: lane (c, h) holds 4 consecutive
+        // channels of row c per accumulator quad (8 bytes); the row pitch of D*2 + 16 bytes keeps the
+        // 8-byte writes and the 16-byte reads below spread over the banks.
+        unsigned char* os = smem + wave * 32 * L::EROW;
 #pragma unroll
         for (int i = 0; i < DB; ++i)
 #pragma unroll
             for (int v4 = 0; v4 < 4; ++v4) {
-                float4 o = make_float4(oacc[i][4 * v4], oacc[i][4 * v4 + 1], oacc[i][4 * v4 + 2], oacc[i][4 * v4 + 3]);
-                *reinterpret_cast<float4*>(os + c * L::OS + 32 * i + 8 * v4 + 4 * h) = o;
+                const f32x4_t o4 = {oacc[i][4 * v4], oacc[i][4 * v4 + 1], oacc[i][4 * v4 + 2], oacc[i][4 * v4 + 3]};
+                const u32x2_t pk = __builtin_bit_cast(u32x2_t, Tag::pack4(o4));      // hardware round-to-nearest-even
+                *reinterpret_cast<u32x2_t*>(os + c * L::EROW + (32 * i + 8 * v4 + 4 * h) * 2) = pk;
             }
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): LDS writes of this wave are visible to it
         const int rows = (hcount - 2 * wave) >= 2 ? 32 : 16;        // this wave's valid rows (whole heads)
         const size_t rid0 = ((size_t)b * A.Hq + hk * A.G + hg0 + 2 * wave) * kM;   // rows are consecutive
-        constexpr int PER_ROW = D / 4;                              // lanes per row, 4 channels each
-        constexpr int RPP = 64 / PER_ROW > 0 ? 64 / PER_ROW : 1;    // rows per pass of the wave
-        const int rsub = lane / PER_ROW, d = (lane % PER_ROW) * 4;
-        for (int r0 = 0; r0 < rows; r0 += 8 * RPP) {
-            float4 o[8];
+        constexpr int PER_ROW = D / 8;                              // lanes per row, 8 channels (16 bytes) each
+        constexpr int RPP = 64 / PER_ROW;                           // rows per pass of the wave
+        const int rsub = lane / PER_ROW, d = (lane % PER_ROW) * 8;
+        uint16_t* dst = A.part_o + ((size_t)split * A.rows_total + rid0) * D + d;
 #pragma unroll
-            for (int u = 0; u < 8; ++u) o[u] = *reinterpret_cast<const float4*>(os + (r0 + u * RPP + rsub) * L::OS + d);
+        for (int r0 = 0; r0 < 32; r0 += 8 * RPP) {
+            u32x4_t o[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) o[u] = *reinterpret_cast<const u32x4_t*>(os + (r0 + u * RPP + rsub) * L::EROW + d * 2);
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 const int r = r0 + u * RPP + rsub;
-                uint2 pk;
-                pk.x = (uint32_t)Tag::cvt(o[u].x) | ((uint32_t)Tag::cvt(o[u].y) << 16);
-                pk.y = (uint32_t)Tag::cvt(o[u].z) | ((uint32_t)Tag::cvt(o[u].w) << 16);
-                if (r < rows) *reinterpret_cast<uint2*>(A.part_o + ((size_t)split * A.rows_total + rid0 + r) * D + d) = pk;
+                if (r < rows) *reinterpret_cast<u32x4_t*>(dst + (size_t)r * D) = o[u];
             }
         }
     }
