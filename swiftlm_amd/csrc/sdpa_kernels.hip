@@ -28,6 +28,8 @@
 // Semantics follow Sources/DFlash/DFlashKernels.swift:737-815 (entry), :563-649
 // (partials: causal rule :614, GQA mapping :575) and :661-720 (combine).
 
+#include <type_traits>
+
 #include "dflash_common.h"
 
 namespace dflash {
@@ -241,63 +243,75 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
         ld_off_k[j] = (uint32_t)row * L::ROWB + (uint32_t)((ld_pos ^ (row & 15)) * 16);
         ld_off_v[j] = (uint32_t)row * L::ROWB + (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
     }
-    auto issue_tile = [&](int t) {
+    // Piece j (of LPW) of tile t: one K and one V load instruction of this wave.
+    auto issue_part = [&](int t, int j) {
         const uint32_t stage_lds = smem_lds + ((t - t_begin) % kStages) * L::STAGE;
         const int key0 = t * kBN;
+        const int rg = (4 * j + wave) * L::RPI;
         if (key0 + kBN <= cache_rows) {          // uniform: whole tile comes from the cache
             const unsigned char* kt = uniform_ptr(kbase + (size_t)key0 * L::ROWB);
             const unsigned char* vt = uniform_ptr(vbase + (size_t)key0 * L::ROWB);
-#pragma unroll
-            for (int j = 0; j < L::LPW; ++j) {
-                const int rg = (4 * j + wave) * L::RPI;
-                async_load_16B(kt, ld_off_k[j], stage_lds + rg * L::ROWB);
-                async_load_16B(vt, ld_off_v[j], stage_lds + L::K_BYTES + rg * L::ROWB);
-            }
+            async_load_16B(kt, ld_off_k[j], stage_lds + rg * L::ROWB);
+            async_load_16B(vt, ld_off_v[j], stage_lds + L::K_BYTES + rg * L::ROWB);
         } else {
             // Tail tile: rows past the end re-read the last key (masked later); with a fused append
             // the block's own 16 rows are taken from k_new / v_new instead of the cache.
-#pragma unroll
-            for (int j = 0; j < L::LPW; ++j) {
-                const int rg = (4 * j + wave) * L::RPI;
-                const int row = rg + ld_rsub;
-                int key = key0 + row;
-                key = key < Nb ? key : Nb - 1;
-                const uint32_t pk = (uint32_t)((ld_pos ^ (row & 15)) * 16);
-                const uint32_t pv = (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
-                const unsigned char* ksrc = key < cache_rows ? kbase + (size_t)key * L::ROWB
-                                                              : knew + (size_t)(key - cache_rows) * L::ROWB;
-                const unsigned char* vsrc = key < cache_rows ? vbase + (size_t)key * L::ROWB
-                                                              : vnew + (size_t)(key - cache_rows) * L::ROWB;
-                async_load_16B_addr(ksrc + pk, stage_lds + rg * L::ROWB);
-                async_load_16B_addr(vsrc + pv, stage_lds + L::K_BYTES + rg * L::ROWB);
-            }
+            const int row = rg + ld_rsub;
+            int key = key0 + row;
+            key = key < Nb ? key : Nb - 1;
+            const uint32_t pk = (uint32_t)((ld_pos ^ (row & 15)) * 16);
+            const uint32_t pv = (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
+            const unsigned char* ksrc = key < cache_rows ? kbase + (size_t)key * L::ROWB
+                                                          : knew + (size_t)(key - cache_rows) * L::ROWB;
+            const unsigned char* vsrc = key < cache_rows ? vbase + (size_t)key * L::ROWB
+                                                          : vnew + (size_t)(key - cache_rows) * L::ROWB;
+            async_load_16B_addr(ksrc + pk, stage_lds + rg * L::ROWB);
+            async_load_16B_addr(vsrc + pv, stage_lds + L::K_BYTES + rg * L::ROWB);
         }
+    };
+    auto issue_tile = [&](int t) {
+#pragma unroll
+        for (int j = 0; j < L::LPW; ++j) issue_part(t, j);
     };
     constexpr int LD_PER_TILE = 2 * L::LPW;      // vmcnt events per tile and wave
 
-    // Tile 0 goes out first, then Q; both are awaited together (one memory round trip), and only
-    // then the rest of the prefetch window is issued, so the first multiply does not wait for
-    // kStages-1 tiles from every CU at once.
+    // Tile 0 goes out first, then Q, then tile 1; tile 0 and Q are awaited together (one memory
+    // round trip).  Q takes the same road as the tiles, HBM -> LDS with 1 KB per wave instruction:
+    // fetched straight into the B-operand layout (16 bytes per lane from 32 rows 512 bytes apart) it
+    // costs 2 us of uncoalesced requests per workgroup.  Each wave parks its own 32 rows, swizzled
+    // like a K tile, in the part of the ring that tiles 2 and 3 will use, reads them back as
+    // operands, and only then (after the barrier) is tile 2 requested.
+    static_assert(kStages >= 4, "Q is parked in stages 2 and 3");
     issue_tile(t_begin);
+    const uint32_t q_park = 2 * L::STAGE + wave * 32 * L::ROWB;
+    if (wave_active) {
+        const int heads_here = (hcount - 2 * wave) >= 2 ? 2 : 1;
+        const unsigned char* qb = reinterpret_cast<const unsigned char*>(A.q) +
+                                  ((size_t)b * A.Hq + hk * A.G + hg0 + 2 * wave) * kM * L::ROWB;
+#pragma unroll
+        for (int j = 0; j < 32 / L::RPI; ++j) {
+            const int row = j * L::RPI + ld_rsub;
+            const int head = (row >> 4) < heads_here ? (row >> 4) : 0;      // an absent head re-reads the first
+            async_load_16B_addr(qb + (size_t)(head * kM + (row & 15)) * L::ROWB + ((ld_pos ^ (row & 15)) * 16),
+                                smem_lds + q_park + j * L::RPI * L::ROWB);
+        }
+    }
+    if (t_begin + 1 < t_end) {
+        issue_tile(t_begin + 1);
+        wait_vmcnt<LD_PER_TILE>();               // tile 0 and Q; tile 1 may still be in flight
+    } else {
+        wait_vmcnt<0>();
+    }
+    asm volatile("" ::: "memory");
 
     // ---- Q as B operands: column c = query row, k-elements 16*s + 8h .. +7 ----
     vec8 qreg[KSTEPS];
-    {
-        const uint16_t* qrow = A.q + row_id * D;
 #pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) {
-            u32x4_t u = {0u, 0u, 0u, 0u};
-            if (row_valid) u = *reinterpret_cast<const u32x4_t*>(qrow + 16 * s + 8 * h);
-            qreg[s] = __builtin_bit_cast(vec8, u);
-        }
-    }
-    // Q must be complete here, and the compiler must know it: it does not see the asynchronous
-    // tile loads, so a Q wait left to it lands on the first MFMA INSIDE the loop as a full
-    // vmcnt(0) drain per tile, which serialises loading and computing.
-    wait_vmcnt<0>();
-#pragma unroll
-    for (int i = 1; i < kStages - 1; ++i)
-        if (t_begin + i < t_end) issue_tile(t_begin + i);
+    for (int s = 0; s < KSTEPS; ++s)
+        qreg[s] = *reinterpret_cast<const vec8*>(smem + q_park + c * L::ROWB + (((2 * s + h) ^ (c & 15)) * 16));
+    __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): Q has left LDS before anyone refills stage 2
+    __builtin_amdgcn_s_barrier();                // tile t_begin is in LDS for all waves; Q is in registers
+    if (t_begin + 2 < t_end) issue_tile(t_begin + 2);
 
     f32x16_t oacc[DB];
 #pragma unroll
@@ -333,13 +347,26 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
     };
     constexpr int kAhead = 4;       // operand reads run this many MFMA steps ahead; sched_barrier pins the order
 
+    // ---- the per-tile work, arranged so that the softmax arithmetic hides behind the MFMAs ----
+    // With one wave per SIMD nothing else fills the VALU while an MFMA runs, and the softmax of a
+    // tile (16 scores per lane: scale, max, 16 quarter-rate exp2, sum, pack) costs about as many
+    // cycles as the tile's 32 MFMAs.  A 32x32x16 MFMA occupies the matrix pipe for 32 cycles after a
+    // 4-cycle issue, and independent VALU instructions of the same wave issue meanwhile.  So each
+    // iteration t runs two blocks:
+    //   phase 1:  S^T(t+1) = K(t+1) Q^T  (MFMA)  with  P(t) = exp2(x(t) - m), row sums, pack  (VALU)
+    //   phase 2:  O^T += V(t)^T P(t)^T   (MFMA)  with  x(t+1) = scale * S^T(t+1), row maximum  (VALU)
+    // where x(t) are tile t's scaled scores.  sched_barrier(0) after every step pins the order.
+    float x[16];                    // scaled (log2 domain) and masked scores of the current tile
+    vec8 pb[2];                     // P^T of the current tile as MFMA operands (two key halves)
+    f32x16_t sacc, sacc1;           // raw scores of the next tile, two accumulation chains
+    float m_pending = -INFINITY;
+
     // S^T = K Q^T of one tile on its own (first tile only).  Two accumulators: a dependent 32x32x16
     // MFMA waits out the pipeline latency of its predecessor, two interleaved chains hide half of it.
-    auto qk_tile = [&](int t, f32x16_t& sc) {
+    auto qk_tile = [&](int t) {
         const unsigned char* ks = stage_of(t);
-        f32x16_t sc1;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) { sc[v] = 0.f; sc1[v] = 0.f; }
+        for (int v = 0; v < 16; ++v) { sacc[v] = 0.f; sacc1[v] = 0.f; }
         vec8 ka[KSTEPS];
 #pragma unroll
         for (int s = 0; s < kAhead; ++s) ka[s] = load_k(ks, s);
@@ -347,37 +374,154 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
 #pragma unroll
         for (int s = 0; s < KSTEPS; s += 2) {
             if (s + kAhead < KSTEPS) { ka[s + kAhead] = load_k(ks, s + kAhead); ka[s + kAhead + 1] = load_k(ks, s + kAhead + 1); }
-            sc = Tag::mfma(ka[s], qreg[s], sc);
-            sc1 = Tag::mfma(ka[s + 1], qreg[s + 1], sc1);
+            sacc = Tag::mfma(ka[s], qreg[s], sacc);
+            sacc1 = Tag::mfma(ka[s + 1], qreg[s + 1], sacc1);
             __builtin_amdgcn_sched_barrier(0);
         }
-#pragma unroll
-        for (int v = 0; v < 16; ++v) sc[v] += sc1[v];
     };
 
-    vec8 pb[2];                     // P^T of the tile whose P V product comes next (two key halves)
-
-    // O^T += V^T P^T of tile t interleaved, MFMA by MFMA, with S^T = K Q^T of tile t+1: the single
-    // dependent Q K^T chain then advances every second issue slot, which is about its latency, and
-    // the eight independent O accumulators fill the slots in between.
-    auto pv_qk_tiles = [&](int t, f32x16_t& sc) {
-        const unsigned char* vs = stage_of(t) + L::K_BYTES;
+    // Phase 1 of iteration t.  Tile t_issue (none if negative) is requested meanwhile, a piece at a time.
+    auto exp_qk = [&](int t, auto with_issue, int t_issue) {
+        constexpr bool kIssue = decltype(with_issue)::value;
+        // the requested tile lies entirely inside the cache: only scalar bases move
+        const uint32_t is_lds = smem_lds + ((t_issue - t_begin) % kStages) * L::STAGE;
+        const unsigned char* is_k = uniform_ptr(kbase + (size_t)t_issue * kBN * L::ROWB);
+        const unsigned char* is_v = uniform_ptr(vbase + (size_t)t_issue * kBN * L::ROWB);
         const unsigned char* ks = stage_of(t + 1);
+        const float m_safe = m_run == -INFINITY ? 0.f : m_run;
+        float psum = 0.f;
+        f32x8_t p0, p1;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) sc[v] = 0.f;
-        vec8 ka[KSTEPS], va[KSTEPS];
+        for (int v = 0; v < 16; ++v) { sacc[v] = 0.f; sacc1[v] = 0.f; }
+        vec8 ka[KSTEPS];
 #pragma unroll
-        for (int s = 0; s < kAhead; ++s) { va[s] = load_v(vs, s); ka[s] = load_k(ks, s); }
+        for (int s = 0; s < kAhead; ++s) ka[s] = load_k(ks, s);
         __builtin_amdgcn_sched_barrier(0);
+        constexpr int PAIRS = KSTEPS / 2;           // MFMA pairs in this block
+        constexpr int EPP = 16 / PAIRS;             // scores handled per pair
+        constexpr int IEV = PAIRS / L::LPW;         // a load piece every IEV pairs
+#pragma unroll
+        for (int s = 0; s < KSTEPS; s += 2) {
+            if (s + kAhead < KSTEPS) { ka[s + kAhead] = load_k(ks, s + kAhead); ka[s + kAhead + 1] = load_k(ks, s + kAhead + 1); }
+            sacc = Tag::mfma(ka[s], qreg[s], sacc);
+            sacc1 = Tag::mfma(ka[s + 1], qreg[s + 1], sacc1);
+            const int pr = s / 2;
+#pragma unroll
+            for (int e = pr * EPP; e < (pr + 1) * EPP; ++e) {
+                const float pe = fast_exp2(x[e] - m_safe);
+                psum += pe;
+                if (e < 8) p0[e] = pe; else p1[e - 8] = pe;
+            }
+            if ((pr + 1) * EPP == 8) pb[0] = Tag::pack(p0);
+            if constexpr (kIssue) {
+                if (pr % IEV == 0) {
+                    const int rg = (4 * (pr / IEV) + wave) * L::RPI;
+                    async_load_16B(is_k, ld_off_k[pr / IEV], is_lds + rg * L::ROWB);
+                    async_load_16B(is_v, ld_off_v[pr / IEV], is_lds + L::K_BYTES + rg * L::ROWB);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        pb[1] = Tag::pack(p1);
+        l_run += psum;
+    };
+
+    // Phase 2 of iteration t: returns the running maximum of x(t+1) over this lane's 16 scores.
+    auto pv_scale = [&](int t) -> float {
+        const unsigned char* vs = stage_of(t) + L::K_BYTES;
+        vec8 va[KSTEPS];
+#pragma unroll
+        for (int s = 0; s < kAhead; ++s) va[s] = load_v(vs, s);
+        __builtin_amdgcn_sched_barrier(0);
+        float mloc = -INFINITY;
+        constexpr int EPS = 16 / KSTEPS;            // scores handled per step
+        constexpr int LAG = 2;                      // steps left to the last score MFMA before its result is read
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
-            if (s + kAhead < KSTEPS) { va[s + kAhead] = load_v(vs, s + kAhead); ka[s + kAhead] = load_k(ks, s + kAhead); }
+            if (s + kAhead < KSTEPS) va[s + kAhead] = load_v(vs, s + kAhead);
             oacc[s % DB] = Tag::mfma(va[s], pb[s / DB], oacc[s % DB]);
-            sc = Tag::mfma(ka[s], qreg[s], sc);
+            if (s >= LAG) {
+#pragma unroll
+                for (int e = (s - LAG) * EPS; e < (s - LAG + 1) * EPS; ++e) {
+                    x[e] = (sacc[e] + sacc1[e]) * A.scale_log2;
+                    mloc = fmaxf(mloc, x[e]);
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
+#pragma unroll
+        for (int e = (KSTEPS - LAG) * EPS; e < 16; ++e) {
+            x[e] = (sacc[e] + sacc1[e]) * A.scale_log2;
+            mloc = fmaxf(mloc, x[e]);
+        }
+        return mloc;
     };
-    auto pv_tile = [&](int t) {     // last tile: nothing left to score
+
+    // Masks on x (tail tiles: the causal rule; MASKED: the additive mask as well) and the row maximum
+    // over both half-waves.  mloc is the maximum of the unmasked scores.
+    auto mask_and_max = [&](int t, float mloc) -> float {
+        const int key0 = t * kBN;
+        const bool need_mask = (key0 + kBN) > (Nb - kM);
+        if (MASKED || need_mask) {                  // uniform
+            const int last_visible = Nb - kM + qi;  // row qi sees keys 0 .. Nb-16+qi
+            float mk[16];
+            if constexpr (MASKED) {
+                const uint16_t* mrow = A.mask + row_id * (size_t)A.N;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    int key = key0 + 8 * (v >> 2) + 4 * h + (v & 3);
+                    key = key < A.N ? key : A.N - 1;               // keys past the end fail the causal rule anyway
+                    mk[v] = row_valid ? Tag::to_f32(mrow[key]) : 0.f;
+                }
+            }
+            mloc = -INFINITY;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                if constexpr (MASKED) {
+                    // -inf (or NaN) drops the key; a finite mask value, however low, keeps it in the softmax
+                    x[v] = mk[v] >= -3.4028234663852886e38f ? fmaxf(fmaf(mk[v], 1.4426950408889634f, x[v]), -3.4028234663852886e38f)
+                                                             : -INFINITY;
+                }
+                const int key = key0 + 8 * (v >> 2) + 4 * h + (v & 3);
+                x[v] = key <= last_visible ? x[v] : -INFINITY;
+                mloc = fmaxf(mloc, x[v]);
+            }
+        }
+        return fmaxf(mloc, __shfl_xor(mloc, 32));
+    };
+
+    // Lazy rescale: the exponent reference m_run only moves when a tile's maximum exceeds it by more
+    // than kRescaleLog2 (P then stays below 2^kRescaleLog2, harmless in fp32/bf16).  Rows that are
+    // still empty take the new reference at once; if rows that already accumulated data must move,
+    // false is returned and the caller rescales the accumulators OUTSIDE the hot loop.  (With the
+    // rescale written inside it the register allocator keeps a VGPR copy of all 128 accumulator
+    // registers and refreshes it on every iteration.)
+    auto accept_max = [&](float ml) -> bool {
+        const bool bump = ml > m_run + kRescaleLog2;        // also true for the first finite maximum
+        if (__builtin_amdgcn_ballot_w64(bump && m_run != -INFINITY) != 0) {
+            m_pending = ml;
+            return false;
+        }
+        if (bump) m_run = ml;
+        return true;
+    };
+
+    // P(t) from x(t) without anything to hide behind (last tile)
+    auto exp_tile = [&]() {
+        const float m_safe = m_run == -INFINITY ? 0.f : m_run;
+        float psum = 0.f;
+        f32x8_t p0, p1;
+#pragma unroll
+        for (int v = 0; v < 8; ++v) {
+            p0[v] = fast_exp2(x[v] - m_safe);
+            p1[v] = fast_exp2(x[v + 8] - m_safe);
+            psum += p0[v] + p1[v];
+        }
+        l_run += psum;
+        pb[0] = Tag::pack(p0);
+        pb[1] = Tag::pack(p1);
+    };
+    auto pv_tile = [&](int t) {
         const unsigned char* vs = stage_of(t) + L::K_BYTES;
         vec8 va[KSTEPS];
 #pragma unroll
@@ -391,95 +535,39 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
         }
     };
 
-    // Scale, causal mask and online softmax (log2 domain) of tile t's raw scores -> pb, m_run, l_run.
-    // Lazy rescale: the exponent reference m_run only moves when the tile's maximum exceeds it by
-    // more than kRescaleLog2 (P then stays below 2^kRescaleLog2, harmless in fp32/bf16).  If rows
-    // that already accumulated data need to move, nothing is changed and false is returned: the
-    // caller rescales the accumulators OUTSIDE the hot loop and calls again.  (With the rescale
-    // written inside the hot loop the register allocator keeps a VGPR copy of all 128 accumulator
-    // registers and refreshes it on every iteration.)
-    float m_pending = -INFINITY;
-    auto softmax_tile = [&](int t, const f32x16_t& sc) -> bool {
-        const int key0 = t * kBN;
-        const bool need_mask = (key0 + kBN) > (Nb - kM);
-        const int last_visible = Nb - kM + qi;     // row qi sees keys 0 .. Nb-16+qi
-        float x[16];
+    // ---- first tile: scores and their maximum ----
+    if (wave_active) {
+        qk_tile(t_begin);
         float mloc = -INFINITY;
-        float mk[16];
-        if constexpr (MASKED) {
-            const uint16_t* mrow = A.mask + row_id * (size_t)A.N;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                int key = key0 + 8 * (v >> 2) + 4 * h + (v & 3);
-                key = key < A.N ? key : A.N - 1;               // keys past the end fail the causal rule anyway
-                mk[v] = row_valid ? Tag::to_f32(mrow[key]) : 0.f;
-            }
-        }
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            x[v] = sc[v] * A.scale_log2;
-            if constexpr (MASKED) {
-                // -inf (or NaN) drops the key; a finite mask value, however low, keeps it in the softmax
-                x[v] = mk[v] >= -3.4028234663852886e38f ? fmaxf(fmaf(mk[v], 1.4426950408889634f, x[v]), -3.4028234663852886e38f)
-                                                         : -INFINITY;
-            }
-            if (need_mask) {
-                const int key = key0 + 8 * (v >> 2) + 4 * h + (v & 3);
-                x[v] = key <= last_visible ? x[v] : -INFINITY;
-            }
+            x[v] = (sacc[v] + sacc1[v]) * A.scale_log2;
             mloc = fmaxf(mloc, x[v]);
         }
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-        const bool bump = mloc > m_run + kRescaleLog2;      // also true for the first finite maximum
-        if (__builtin_amdgcn_ballot_w64(bump && m_run != -INFINITY) != 0) {
-            m_pending = mloc;
-            return false;
-        }
-        const float m_new = bump ? mloc : m_run;            // a bump here starts from an empty row
-        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-        m_run = m_new;
-        float psum = 0.f;
-        f32x8_t p0, p1;
-#pragma unroll
-        for (int v = 0; v < 8; ++v) {
-            p0[v] = fast_exp2(x[v] - m_safe);
-            p1[v] = fast_exp2(x[v + 8] - m_safe);
-            psum += p0[v] + p1[v];
-        }
-        l_run += psum;
-        pb[0] = Tag::pack(p0);
-        pb[1] = Tag::pack(p1);
-        return true;
-    };
-
-    // ---- first tile: scores and softmax; afterwards every iteration multiplies tile t by V while it
-    // scores tile t+1 ----
-    __builtin_amdgcn_s_barrier();                  // tile t_begin (awaited together with Q) is in LDS for all waves
-    f32x16_t sacc;
-    if (wave_active) {
-        qk_tile(t_begin, sacc);
-        softmax_tile(t_begin, sacc);               // rows are empty: cannot ask for a rescale
+        accept_max(mask_and_max(t_begin, mloc));   // rows are empty: cannot ask for a rescale
     }
     int t = t_begin;
     const int t_last = t_end - 1;
-    bool redo = false;                             // the MFMA part of iteration t is done, only the softmax is repeated
     while (t < t_last) {
         bool jumped = false;
         for (; t < t_last; ++t) {
-            if (!redo) {
-                // tile t+1 has landed once at most (tiles issued after it) * LD_PER_TILE loads are outstanding
-                const int later = (t_last - 1 - t) < (kStages - 3) ? (t_last - 1 - t) : (kStages - 3);
-                if (later >= 2) wait_vmcnt<2 * LD_PER_TILE>();
-                else if (later == 1) wait_vmcnt<LD_PER_TILE>();
-                else wait_vmcnt<0>();
-                __builtin_amdgcn_s_barrier();      // tile t+1 is in LDS for everyone; everyone is done with tile t-1
-                if (t + kStages - 1 < t_end) issue_tile(t + kStages - 1);   // refills the stage tile t-1 used
-                if (wave_active) pv_qk_tiles(t, sacc);
-            }
-            redo = false;
-            if (wave_active && !softmax_tile(t + 1, sacc)) {
-                jumped = true;
-                break;
+            // tile t+1 has landed once at most (tiles issued after it) * LD_PER_TILE loads are outstanding
+            const int later = (t_last - 1 - t) < (kStages - 3) ? (t_last - 1 - t) : (kStages - 3);
+            if (later >= 2) wait_vmcnt<2 * LD_PER_TILE>();
+            else if (later == 1) wait_vmcnt<LD_PER_TILE>();
+            else wait_vmcnt<0>();
+            __builtin_amdgcn_s_barrier();          // tile t+1 is in LDS for everyone; everyone is done with tile t-1
+            const int t_issue = (t + kStages - 1 < t_end) ? t + kStages - 1 : -1;   // refills the stage tile t-1 used
+            const bool spread = t_issue >= 0 && (t_issue + 1) * kBN <= cache_rows;  // requested between the MFMAs
+            if (t_issue >= 0 && !(spread && wave_active)) issue_tile(t_issue);      // tail tile, or a wave without rows
+            if (wave_active) {
+                if (spread) exp_qk(t, std::true_type{}, t_issue);
+                else exp_qk(t, std::false_type{}, 0);
+                const float mloc = pv_scale(t);
+                if (!accept_max(mask_and_max(t + 1, mloc))) {
+                    jumped = true;
+                    break;
+                }
             }
         }
         if (jumped) {                              // cold: move the exponent reference of the rows that jumped
@@ -491,10 +579,13 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
             for (int i = 0; i < DB; ++i)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
-            redo = true;
+            ++t;                                   // x already holds tile t+1's scores
         }
     }
-    if (wave_active) pv_tile(t_last);              // its scores were taken one iteration earlier
+    if (wave_active) {                             // last tile: nothing left to score
+        exp_tile();
+        pv_tile(t_last);
+    }
     __syncthreads();          // the tile buffers are free for the epilogue
 
     // ---- epilogue: partial statistics and O rows (through LDS for coalesced stores) ----
@@ -627,6 +718,15 @@ static int choose_splits(int B, int Hk, int groups_per_kv, int N) {
     const int cus = num_compute_units();
     const int per = B * Hk * groups_per_kv;
     int S = (cus + per - 1) / per;
+    // Every split pays a fixed price (its partial rows, written once and read back by the combine
+    // kernel, are as large as 4 tiles of K/V), so a short context is not spread thinner than
+    // kMinTilesPerSplit tiles per workgroup.
+    // kMinTilesPerSplit tiles per workgroup, unless that leaves fewer than kMinSplits workgroups
+    // per KV head (then latency, not the partials, is what counts).
+    constexpr int kMinTilesPerSplit = 4, kMinSplits = 32;
+    int floor_s = nt / kMinTilesPerSplit;
+    if (floor_s < kMinSplits) floor_s = kMinSplits;
+    if (S > floor_s) S = floor_s;
     if (S > nt) S = nt;
     if (S > kMaxSplits) S = kMaxSplits;
     if (S < 1) S = 1;
