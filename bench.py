@@ -147,7 +147,7 @@ def main():
     _lib.check(lib.dflash_init(), "dflash_init")
 
     K, W = args.steps, args.warmup
-    brk_steps = min(max(K, 1), 16)                 # eager pass with per-kernel event brackets
+    brk_steps = min(max(K, 1), 16)                 # eager pass with events attached to the kernels
     total = 2 + W + K + brk_steps
     cfg = StackConfig(context=args.context, max_steps=total + 2)
     stack = HybridVerifyStack(cfg, seed=0)

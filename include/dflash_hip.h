@@ -235,10 +235,11 @@ int dflash_kv_append(void* stream, void* k_cache, void* v_cache, const void* k_n
 /* ------------------------------------------------------------------------
  * Measurement hook (no counterpart in the reference, whose bench times whole
  * calls from the host: Sources/DFlashKernelBench/main.swift:33-57).  Arms the
- * calling thread so that the NEXT launch of the named kernel is bracketed by
- * hipEventRecord(start_event) / hipEventRecord(stop_event) on the launch stream;
- * the arming is consumed by that launch.  Events are hipEvent_t passed as void*,
- * created and read by the caller.
+ * calling thread so that the NEXT launch of the named kernel carries the two
+ * events on its own dispatch (hipExtLaunchKernelGGL): their elapsed time is the
+ * kernel's begin-to-end duration on the launch stream, as a profiler's kernel
+ * trace reports it.  The arming is consumed by that launch.  Events are
+ * hipEvent_t passed as void*, created and read by the caller.
  * ---------------------------------------------------------------------- */
 #define DFLASH_KERNEL_SDPA_PARTIAL 0
 #define DFLASH_KERNEL_SDPA_COMBINE 1
