@@ -64,8 +64,9 @@ struct ReplayArgs {
 constexpr int kReplayChunk = 32;  // steps staged in LDS at a time (16 for Dk = 256)
 
 // One thread owns 4 consecutive key channels of NR state rows.  DK/4 threads
-// span a row, so a 256-thread workgroup covers RPP = 1024/DK rows per pass and
-// NR passes.  Grid: x = Dv tiles, y = b*Hv + hv, z = layer.
+// span a row, so a 256-thread workgroup covers RPP = floor(1024/DK) rows per pass
+// and NR passes (when DK/4 does not divide 256 the last few threads only help
+// with staging).  Grid: x = Dv tiles, y = b*Hv + hv, z = layer.
 template <typename StateT, bool VEC_G, int DK, int NR>
 __global__ __launch_bounds__(kThreads) void tape_replay_kernel(ReplayBatch P, ReplayArgs A) {
     constexpr int TPR = DK / 4;
@@ -85,7 +86,8 @@ __global__ __launch_bounds__(kThreads) void tape_replay_kernel(ReplayBatch P, Re
     const int row0 = blockIdx.x * ROWS;
     const int tid = threadIdx.x;
     const int c4 = (tid % TPR) * 4;
-    const int rsub = tid / TPR;
+    const bool owner = tid < RPP * TPR;            // false only for the spare threads of an odd TPR
+    const int rsub = owner ? tid / TPR : 0;
 
     int n = A.steps_dev ? *A.steps_dev : A.steps;
     n = n < 0 ? 0 : (n > A.T_tape ? A.T_tape : n);
@@ -101,7 +103,7 @@ __global__ __launch_bounds__(kThreads) void tape_replay_kernel(ReplayBatch P, Re
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
         const int r = row0 + rsub + RPP * i;
-        s[i] = r < A.Dv ? load4(s_in + (size_t)r * DK + c4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        s[i] = (owner && r < A.Dv) ? load4(s_in + (size_t)r * DK + c4) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 
     for (int t0 = 0; t0 < n; t0 += TC) {
@@ -146,7 +148,7 @@ __global__ __launch_bounds__(kThreads) void tape_replay_kernel(ReplayBatch P, Re
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
         const int r = row0 + rsub + RPP * i;
-        if (r < A.Dv) store4(s_out + (size_t)r * DK + c4, s[i]);
+        if (owner && r < A.Dv) store4(s_out + (size_t)r * DK + c4, s[i]);
     }
 }
 
@@ -179,12 +181,18 @@ static int launch_replay_state(hipStream_t st, const ReplayBatch& P, const Repla
     switch (Dk) {
         DFLASH_REPLAY_CASE(32)
         DFLASH_REPLAY_CASE(64)
+        DFLASH_REPLAY_CASE(96)
         DFLASH_REPLAY_CASE(128)
+        DFLASH_REPLAY_CASE(160)
+        DFLASH_REPLAY_CASE(192)
+        DFLASH_REPLAY_CASE(224)
         DFLASH_REPLAY_CASE(256)
         default: break;
     }
 #undef DFLASH_REPLAY_CASE
-    set_error("tape replay: Dk=%d is not one of 32, 64, 128, 256", Dk);
+    // the reference's Metal kernels take every multiple of 32 (DFlashKernels.swift:271-273); beyond 256 the
+    // caller is told to use its general path
+    set_error("tape replay: Dk=%d is not a multiple of 32 in [32, 256]", Dk);
     return DFLASH_UNSUPPORTED;
 }
 
@@ -707,12 +715,16 @@ static int launch_gdn_state(hipStream_t st, const GdnArgs& A, int B, int g_ndim,
     switch (Dk) {
         DFLASH_GDN_CASE(32, 8)
         DFLASH_GDN_CASE(64, 16)
+        DFLASH_GDN_CASE(96, 8)
         DFLASH_GDN_CASE(128, 16)
+        DFLASH_GDN_CASE(160, 8)
+        DFLASH_GDN_CASE(192, 16)
+        DFLASH_GDN_CASE(224, 8)
         DFLASH_GDN_CASE(256, 16)
         default: break;
     }
 #undef DFLASH_GDN_CASE
-    set_error("gated delta: Dk=%d is not one of 32, 64, 128, 256", Dk);
+    set_error("gated delta: Dk=%d is not a multiple of 32 in [32, 256]", Dk);
     return DFLASH_UNSUPPORTED;
 }
 

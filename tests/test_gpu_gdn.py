@@ -50,6 +50,10 @@ SHAPES = [
     ("ragged_dv", 2, 5, 2, 6, 128, 40),
     ("dk32", 1, 7, 2, 4, 32, 24),
     ("dk256", 1, 6, 1, 2, 256, 64),
+    ("dk96", 1, 9, 2, 4, 96, 40),        # DK/4 = 24 threads per row does not divide the workgroup
+    ("dk160", 2, 5, 1, 3, 160, 16),
+    ("dk192", 1, 18, 2, 2, 192, 48),
+    ("dk224", 1, 4, 1, 2, 224, 24),
     ("long_T", 1, 40, 2, 4, 64, 32),
 ]
 
