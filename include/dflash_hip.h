@@ -205,6 +205,32 @@ int dflash_accept_commit(void* stream, const uint32_t* verify_ids, const uint32_
                          int32_t* start_inout, int32_t* out4);
 
 /* ------------------------------------------------------------------------
+ * Greedy tokens over the verify logits.  dflash_greedy_tokens_with_mask replaces
+ * DFlashRuntime.greedyTokensWithMask (DFlashRuntime.swift:118-128):
+ *   tokens_out[t] = argmax_v where(suppress_mask[v], (dtype)(-1e9), logits[t, v])
+ * with the lowest index winning a tie (the array library's argMax is not in the
+ * reference tree; first-index is what its callers' tests and numpy/torch agree
+ * on).  logits [T, V] row-major in `dtype` (f32/bf16/f16); suppress_mask NULL or
+ * uint8 [V], non-zero = suppressed (buildSuppressTokenMask, :105-115).
+ *
+ * dflash_greedy_accept_commit does that and dflash_accept_commit's bookkeeping in
+ * one call (the cycle's :513-547; two launches: per-chunk maxima, then one
+ * workgroup that reduces them and does the bookkeeping): posterior_out [T] receives
+ * the greedy tokens, out4 / start_inout are as for dflash_accept_commit with V == T.
+ *
+ * workspace: at least dflash_greedy_workspace_bytes(T, V) bytes, 256-byte
+ * aligned; contents are undefined before and after.
+ * ---------------------------------------------------------------------- */
+size_t dflash_greedy_workspace_bytes(int T, int V);
+int dflash_greedy_tokens_with_mask(void* stream, const void* logits, int dtype, int T, int V,
+                                   const uint8_t* suppress_mask, uint32_t* tokens_out,
+                                   void* workspace, size_t workspace_bytes);
+int dflash_greedy_accept_commit(void* stream, const void* logits, int dtype, int T, int V,
+                                const uint8_t* suppress_mask, const uint32_t* verify_ids,
+                                int32_t* start_inout, int32_t* out4, uint32_t* posterior_out,
+                                void* workspace, size_t workspace_bytes);
+
+/* ------------------------------------------------------------------------
  * Conv-state rebuild after rollback.  Replaces
  * RecurrentRollbackCache.rebuildConvState (Sources/DFlash/
  * RecurrentRollbackCache.swift:139-158):
@@ -245,7 +271,8 @@ int dflash_kv_append(void* stream, void* k_cache, void* v_cache, const void* k_n
 #define DFLASH_KERNEL_SDPA_COMBINE 1
 #define DFLASH_KERNEL_GDN_FORWARD 2
 #define DFLASH_KERNEL_TAPE_REPLAY 3
-#define DFLASH_KERNEL_COUNT 4
+#define DFLASH_KERNEL_GREEDY_PARTIAL 4
+#define DFLASH_KERNEL_COUNT 5
 int dflash_profile_next_launch(int kernel_id, void* start_event, void* stop_event);
 
 #ifdef __cplusplus

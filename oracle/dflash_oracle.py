@@ -184,6 +184,34 @@ def gated_delta_ops_with_tape(q, k, v, g, beta, state, mask=None, *, dtype=np.fl
 # ----------------------------------------------------------------------------
 
 
+def build_suppress_token_mask(vocab_size: int, suppress_token_ids):
+    """Boolean [vocab] mask of the in-range ids, or None when there are none
+    (DFlashRuntime.swift:105-115)."""
+    ids = sorted({int(i) for i in (suppress_token_ids or []) if 0 <= int(i) < vocab_size})
+    if not ids:
+        return None
+    mask = np.zeros(vocab_size, dtype=bool)
+    mask[ids] = True
+    return mask
+
+
+def greedy_tokens_with_mask(logits, suppress_token_mask=None, *, dtype="f32"):
+    """``argmax(where(mask, -1e9 as logits.dtype, logits), axis=-1)`` as uint32
+    (DFlashRuntime.swift:118-128).  ``dtype`` names the logits' type: the floor is
+    -1e9 ROUNDED to it (bf16: -999292928).  The first index wins a tie (numpy's
+    argmax rule; the array library's own argMax is not in the reference tree)."""
+    x = np.asarray(logits, dtype=np.float32)
+    if suppress_token_mask is not None:
+        floor = np.float32(-1e9)
+        if dtype == "bf16":
+            floor = round_to_bf16(np.array([floor], np.float32))[0]
+        elif dtype == "f16":
+            with np.errstate(over="ignore"):
+                floor = np.float32(np.float16(floor))       # -inf: -1e9 overflows float16
+        x = np.where(np.asarray(suppress_token_mask, dtype=bool), floor, x)
+    return np.argmax(x, axis=-1).astype(np.uint32)
+
+
 def match_acceptance_length(drafted, posterior) -> int:
     """Number of leading positions where drafted == posterior.
 

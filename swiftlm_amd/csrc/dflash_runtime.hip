@@ -7,6 +7,8 @@
 
 #include <mutex>
 
+#include <type_traits>
+
 #include "dflash_common.h"
 
 namespace dflash {
@@ -96,6 +98,133 @@ __global__ __launch_bounds__(64) void accept_commit_kernel(const uint32_t* verif
     }
 }
 
+// ---- greedy tokens over the verify logits, fused with the acceptance ---------
+
+// DFlashRuntime.greedyTokensWithMask (DFlashRuntime.swift:118-128): argmax over the vocabulary of
+// where(mask, -1e9 rounded to the logits' type, logits); the first index wins a tie.  HBM-bound
+// (T x V logits read once).  Two launches: greedy_partial_kernel (grid x = chunks of kArgmaxChunk
+// vocabulary entries, y = row) leaves a (best value, best index) pair per workgroup in the
+// workspace; greedy_finish_kernel (one workgroup) reduces them, writes posterior[T] and, when asked
+// to, does the cycle's acceptance bookkeeping (accept_commit_kernel above).  A single launch with a
+// "last workgroup finishes" ticket was measured slower: the device-scope fences and the atomic it
+// needs add more dependent memory round trips than the second launch costs.
+constexpr int kArgmaxThreads = 256;
+constexpr int kArgmaxChunk = 8192;
+constexpr int kArgmaxMaxRows = 1024;
+constexpr int kArgmaxMaxPartials = 4096;   // T * chunks the last workgroup can hold in LDS
+
+struct GreedyArgs {
+    const void* logits;            // [T, V]
+    const uint8_t* suppress;       // [V] non-zero = suppressed, or null
+    const uint32_t* verify_ids;    // [T], or null: tokens only
+    int32_t* start_inout;
+    int32_t* out4;
+    uint32_t* posterior;           // [T]
+    float* part_val;               // [T, chunks]
+    int32_t* part_idx;             // [T, chunks]
+    int T, V, chunks;
+};
+
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
+
+template <typename Elem>
+__global__ __launch_bounds__(kArgmaxThreads) void greedy_partial_kernel(GreedyArgs A) {
+    __shared__ float val_s[kArgmaxThreads / 64];
+    __shared__ int idx_s[kArgmaxThreads / 64];
+    const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+    const Elem* lrow = reinterpret_cast<const Elem*>(A.logits) + (size_t)row * A.V;
+    const float floor_v = to_float(from_float<Elem>(-1e9f));      // MLXArray(-1e9, dtype: logits.dtype) (:124)
+    const int v0 = chunk * kArgmaxChunk;
+    const int v1 = (v0 + kArgmaxChunk) < A.V ? (v0 + kArgmaxChunk) : A.V;
+
+    float best = -INFINITY;
+    int besti = 0x7fffffff;
+    constexpr int VEC = 16 / sizeof(Elem);                        // elements per 16-byte load
+    typedef typename std::conditional<VEC == 8, uint64_t, uint32_t>::type MaskWord;   // VEC mask bytes at once
+    const bool aligned = ((size_t)row * A.V * sizeof(Elem)) % 16 == 0 && (uintptr_t)A.logits % 16 == 0 &&
+                         (uintptr_t)A.suppress % sizeof(MaskWord) == 0;
+    if (aligned) {
+        for (int i = v0 + tid * VEC; i < v1; i += kArgmaxThreads * VEC) {
+            if (i + VEC <= v1) {
+                Elem e[VEC];
+                *reinterpret_cast<uint4*>(e) = *reinterpret_cast<const uint4*>(lrow + i);
+                const MaskWord mw = A.suppress ? *reinterpret_cast<const MaskWord*>(A.suppress + i) : (MaskWord)0;
+#pragma unroll
+                for (int u = 0; u < VEC; ++u) {
+                    float x = to_float(e[u]);
+                    if ((mw >> (8 * u)) & 0xff) x = floor_v;
+                    if (x > best) { best = x; besti = i + u; }    // ascending indices: '>' keeps the first maximum
+                }
+            } else {
+                for (int j = i; j < v1; ++j) {
+                    float x = to_float(lrow[j]);
+                    if (A.suppress && A.suppress[j]) x = floor_v;
+                    if (x > best) { best = x; besti = j; }
+                }
+            }
+        }
+    } else {
+        for (int j = v0 + tid; j < v1; j += kArgmaxThreads) {
+            float x = to_float(lrow[j]);
+            if (A.suppress && A.suppress[j]) x = floor_v;
+            if (x > best) { best = x; besti = j; }
+        }
+    }
+    for (int o = 32; o >= 1; o >>= 1) {
+        const float ov = __shfl_xor(best, o);
+        const int oi = __shfl_xor(besti, o);
+        if (better(ov, oi, best, besti)) { best = ov; besti = oi; }
+    }
+    if ((tid & 63) == 0) { val_s[tid >> 6] = best; idx_s[tid >> 6] = besti; }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < kArgmaxThreads / 64; ++w)
+            if (better(val_s[w], idx_s[w], best, besti)) { best = val_s[w]; besti = idx_s[w]; }
+        A.part_val[row * A.chunks + chunk] = best;
+        A.part_idx[row * A.chunks + chunk] = besti;
+    }
+}
+
+__global__ __launch_bounds__(kArgmaxThreads) void greedy_finish_kernel(GreedyArgs A) {
+    const int tid = threadIdx.x;
+    // every thread fetches partials at once (one memory round trip), then one wave reduces them per
+    // row out of LDS
+    __shared__ float pv_s[kArgmaxMaxPartials];
+    __shared__ int pi_s[kArgmaxMaxPartials];
+    const int total = A.T * A.chunks;
+    for (int p = tid; p < total; p += kArgmaxThreads) {
+        pv_s[p] = A.part_val[p];
+        pi_s[p] = A.part_idx[p];
+    }
+    __syncthreads();
+    if (tid >= 64) return;
+    __shared__ uint32_t post_s[kArgmaxMaxRows];
+    for (int r = tid; r < A.T; r += 64) {
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int c = 0; c < A.chunks; ++c)
+            if (better(pv_s[r * A.chunks + c], pi_s[r * A.chunks + c], bv, bi)) { bv = pv_s[r * A.chunks + c]; bi = pi_s[r * A.chunks + c]; }
+        // a row of NaNs never compares greater than anything: token 0, like a scan that starts at index 0
+        const uint32_t tok = bi == 0x7fffffff ? 0u : (uint32_t)bi;
+        post_s[r] = tok;
+        A.posterior[r] = tok;
+    }
+    if (A.verify_ids) {
+        __builtin_amdgcn_s_waitcnt(0xc07f);                       // lgkmcnt(0): this wave's LDS writes have landed
+        __builtin_amdgcn_wave_barrier();
+        const int acc = A.T > 1 ? leading_matches(A.verify_ids + 1, post_s, A.T - 1) : 0;
+        if (tid == 0) {
+            const int commit = 1 + acc;
+            A.out4[0] = acc;
+            A.out4[1] = commit;
+            A.out4[2] = (int32_t)post_s[acc];
+            int start = commit;
+            if (A.start_inout) { start += *A.start_inout; *A.start_inout = start; }
+            A.out4[3] = start;
+        }
+    }
+}
+
 // ---- conv-state rebuild ----------------------------------------------------
 
 // out[b, j, :] = concat(snapshot [B,keep,C], qkv [B,T,C])[b, s + j, :], 16-byte pieces.
@@ -169,6 +298,71 @@ extern "C" int dflash_accept_commit(void* stream, const uint32_t* verify_ids, co
                        start_inout, out4);
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
+}
+
+static size_t greedy_ws_layout(int T, int V, size_t* off_idx) {
+    const size_t chunks = (size_t)(V + kArgmaxChunk - 1) / kArgmaxChunk;
+    size_t o = (size_t)T * chunks * sizeof(float);
+    o = (o + 255) & ~(size_t)255;
+    *off_idx = o;
+    o += (size_t)T * chunks * sizeof(int32_t);
+    return (o + 255) & ~(size_t)255;
+}
+
+extern "C" size_t dflash_greedy_workspace_bytes(int T, int V) {
+    if (T <= 0 || V <= 0) return 0;
+    size_t a;
+    return greedy_ws_layout(T, V, &a);
+}
+
+static int greedy_common(void* stream, const void* logits, int dtype, int T, int V, const uint8_t* suppress,
+                         const uint32_t* verify_ids, int32_t* start_inout, int32_t* out4, uint32_t* posterior,
+                         void* workspace, size_t workspace_bytes) {
+    int rc = ensure_init();
+    if (rc) return rc;
+    DFLASH_REQUIRE(logits && posterior && T >= 1 && V >= 1, "greedy tokens: bad arguments");
+    DFLASH_SUPPORTED(T <= kArgmaxMaxRows, "greedy tokens: T=%d rows exceed %d", T, kArgmaxMaxRows);
+    DFLASH_SUPPORTED((long)T * ((V + kArgmaxChunk - 1) / kArgmaxChunk) <= kArgmaxMaxPartials,
+                     "greedy tokens: T=%d x V=%d needs more than %d partial results", T, V, kArgmaxMaxPartials);
+    DFLASH_SUPPORTED(dtype == DFLASH_F32 || dtype == DFLASH_BF16 || dtype == DFLASH_F16, "greedy tokens: bad dtype %d", dtype);
+    size_t oi;
+    const size_t need = greedy_ws_layout(T, V, &oi);
+    DFLASH_REQUIRE(workspace && workspace_bytes >= need, "greedy tokens: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    DFLASH_REQUIRE((uintptr_t)workspace % 256 == 0, "greedy tokens: workspace must be 256-byte aligned");
+    GreedyArgs A;
+    A.logits = logits; A.suppress = suppress; A.verify_ids = verify_ids; A.start_inout = start_inout; A.out4 = out4;
+    A.posterior = posterior;
+    A.part_val = (float*)workspace;
+    A.part_idx = (int32_t*)((char*)workspace + oi);
+    A.T = T; A.V = V; A.chunks = (V + kArgmaxChunk - 1) / kArgmaxChunk;
+    dim3 grid(A.chunks, T);
+    hipStream_t st = (hipStream_t)stream;
+    {
+        LaunchBracket br(DFLASH_KERNEL_GREEDY_PARTIAL, st);
+        if (dtype == DFLASH_F32) br.launch(greedy_partial_kernel<float>, grid, dim3(kArgmaxThreads), 0, A);
+        else if (dtype == DFLASH_BF16) br.launch(greedy_partial_kernel<bf16_t>, grid, dim3(kArgmaxThreads), 0, A);
+        else br.launch(greedy_partial_kernel<f16_t>, grid, dim3(kArgmaxThreads), 0, A);
+    }
+    DFLASH_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(greedy_finish_kernel, dim3(1), dim3(kArgmaxThreads), 0, st, A);
+    DFLASH_HIP_TRY(hipGetLastError());
+    return DFLASH_OK;
+}
+
+extern "C" int dflash_greedy_tokens_with_mask(void* stream, const void* logits, int dtype, int T, int V,
+                                              const uint8_t* suppress_mask, uint32_t* tokens_out, void* workspace,
+                                              size_t workspace_bytes) {
+    return greedy_common(stream, logits, dtype, T, V, suppress_mask, nullptr, nullptr, nullptr, tokens_out, workspace,
+                         workspace_bytes);
+}
+
+extern "C" int dflash_greedy_accept_commit(void* stream, const void* logits, int dtype, int T, int V,
+                                           const uint8_t* suppress_mask, const uint32_t* verify_ids,
+                                           int32_t* start_inout, int32_t* out4, uint32_t* posterior_out,
+                                           void* workspace, size_t workspace_bytes) {
+    DFLASH_REQUIRE(verify_ids && out4, "greedy accept: null pointer");
+    return greedy_common(stream, logits, dtype, T, V, suppress_mask, verify_ids, start_inout, out4, posterior_out,
+                         workspace, workspace_bytes);
 }
 
 extern "C" int dflash_rebuild_conv_state(void* stream, const void* snapshot_conv, const void* tape_qkv, void* out, int B,

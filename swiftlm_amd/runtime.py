@@ -16,7 +16,7 @@ from typing import List, Sequence
 import torch
 
 from . import _lib
-from .dflash_kernels import _ptr, _stream
+from .dflash_kernels import _code, _ptr, _stream
 from .rollback_cache import RecurrentRollbackCache, _NativeCache, _RollbackCache
 
 
@@ -29,7 +29,70 @@ class AcceptResult:
     start: int
 
 
+_greedy_ws = {}
+
+
+def _greedy_workspace(T: int, V: int, device) -> torch.Tensor:
+    """One scratch tensor per (T, V, device, stream): launches sharing it must not overlap, which
+    one stream guarantees."""
+    key = (T, V, str(device), int(_stream().value or 0))
+    ws = _greedy_ws.get(key)
+    if ws is None:
+        need = int(_lib.load().dflash_greedy_workspace_bytes(T, V))
+        ws = torch.empty(need, dtype=torch.uint8, device=device)
+        _greedy_ws[key] = ws
+    return ws
+
+
 class DFlashRuntime:
+    # -- token utilities -------------------------------------------------------------
+    @staticmethod
+    def build_suppress_token_mask(vocab_size: int, suppress_token_ids, device="cuda"):
+        """``buildSuppressTokenMask(vocabSize:suppressTokenIDs:)`` (DFlashRuntime.swift:105-115):
+        uint8 [vocab] on the device, or None when no id is in range."""
+        ids = sorted({int(i) for i in (suppress_token_ids or []) if 0 <= int(i) < vocab_size})
+        if not ids:
+            return None
+        mask = torch.zeros(vocab_size, dtype=torch.uint8)
+        mask[ids] = 1
+        return mask.to(device)
+
+    @staticmethod
+    def greedy_tokens_with_mask(logits: torch.Tensor, suppress_token_mask=None) -> torch.Tensor:
+        """``greedyTokensWithMask(logits:suppressTokenMask:)`` (DFlashRuntime.swift:118-128):
+        logits [T, V] -> int32 [T] holding the reference's uint32 token ids."""
+        if not logits.is_cuda or logits.dim() != 2:
+            raise _lib.DFlashError("greedy_tokens_with_mask: logits must be a [T, V] tensor on the GPU")
+        logits = logits.contiguous()
+        T, V = logits.shape
+        m = None if suppress_token_mask is None else suppress_token_mask.to(torch.uint8).contiguous()
+        out = torch.empty(T, dtype=torch.int32, device=logits.device)
+        ws = _greedy_workspace(T, V, logits.device)
+        rc = _lib.load().dflash_greedy_tokens_with_mask(_stream(), _ptr(logits), _code(logits), T, V, _ptr(m), _ptr(out),
+                                                        _ptr(ws), ws.numel())
+        _lib.check(rc, "greedy_tokens_with_mask")
+        return out
+
+    @staticmethod
+    def greedy_accept_commit(logits: torch.Tensor, suppress_token_mask, verify_ids: torch.Tensor, start: int):
+        """The cycle's greedy tokens, acceptance length and commit bookkeeping in one call
+        (DFlashRuntime.swift:513-547): returns (AcceptResult, posterior int32 [T])."""
+        logits = logits.contiguous()
+        T, V = logits.shape
+        if int(verify_ids.shape[0]) != T:
+            raise _lib.DFlashError("greedy_accept_commit: one logits row per verify position")
+        m = None if suppress_token_mask is None else suppress_token_mask.to(torch.uint8).contiguous()
+        v = verify_ids.to(torch.int32).contiguous()
+        post = torch.empty(T, dtype=torch.int32, device=logits.device)
+        out = torch.empty(4, dtype=torch.int32, device=logits.device)
+        st = torch.tensor([start], dtype=torch.int32, device=logits.device)
+        ws = _greedy_workspace(T, V, logits.device)
+        rc = _lib.load().dflash_greedy_accept_commit(_stream(), _ptr(logits), _code(logits), T, V, _ptr(m), _ptr(v), _ptr(st),
+                                                     _ptr(out), _ptr(post), _ptr(ws), ws.numel())
+        _lib.check(rc, "greedy_accept_commit")
+        a, c, s, n = out.tolist()
+        return AcceptResult(a, c, s, n), post
+
     # -- acceptance ----------------------------------------------------------------
     @staticmethod
     def match_acceptance_length(drafted_tokens: torch.Tensor, posterior_tokens: torch.Tensor) -> torch.Tensor:

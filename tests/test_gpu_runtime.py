@@ -217,3 +217,58 @@ def test_snapshot_cache_restores_pre_verify_state(gpu_lib):
     c[0], c[1] = conv * 2, state * 2
     c.rollback(5)
     assert c[0] is conv and c[1] is state and not c.is_armed
+
+
+# ---- greedy tokens + fused acceptance (DFlashRuntime.swift:118-128, :513-547) ----
+
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("V", [151936, 8192, 1000, 37])
+def test_greedy_tokens_with_mask_matches_oracle(gpu_lib, dt, V):
+    import torch
+    from swiftlm_amd import DFlashRuntime
+    tdt = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[dt]
+    T = 16
+    g = torch.Generator(device="cuda").manual_seed(V)
+    logits = (4 * torch.randn(T, V, generator=g, device="cuda")).to(tdt)
+    ids = [0, 5, V - 1, V + 3, -2] + list(range(10, min(V, 30)))
+    # make the unmasked winner of some rows a suppressed token, and plant exact ties
+    logits[0, 5] = 100.0
+    logits[1, V - 1] = 100.0
+    logits[2, 7] = 90.0
+    logits[2, V // 2] = 90.0
+    logits[3, :] = 1.0
+    host_logits = logits.float().cpu().numpy()
+    for ids_case in (None, ids):
+        mask_o = O.build_suppress_token_mask(V, ids_case)
+        mask_d = DFlashRuntime.build_suppress_token_mask(V, ids_case)
+        assert (mask_o is None) == (mask_d is None)
+        got = DFlashRuntime.greedy_tokens_with_mask(logits, mask_d)
+        torch.cuda.synchronize()
+        want = O.greedy_tokens_with_mask(host_logits, mask_o, dtype=dt)
+        np.testing.assert_array_equal(got.cpu().numpy().astype(np.uint32), want)
+
+
+def test_greedy_accept_commit_equals_two_steps(gpu_lib):
+    """One call = greedyTokensWithMask + matchAcceptanceLength + the commit bookkeeping; repeated
+    calls reuse the workspace."""
+    import torch
+    from swiftlm_amd import DFlashRuntime
+    T, V = 16, 151936
+    g = torch.Generator(device="cuda").manual_seed(1)
+    mask = DFlashRuntime.build_suppress_token_mask(V, [1, 2, 3])
+    start = 1000
+    for acc in (0, 3, 15, 7):
+        logits = torch.randn(T, V, generator=g, device="cuda").bfloat16()
+        post = O.greedy_tokens_with_mask(logits.float().cpu().numpy(), O.build_suppress_token_mask(V, [1, 2, 3]), dtype="bf16")
+        verify = np.empty(T, np.int64)
+        verify[0] = 42
+        verify[1:] = post[:-1]
+        if acc < T - 1:
+            verify[1 + acc] = (int(post[acc]) + 1) % V          # first mismatch at draft position acc
+        res, post_d = DFlashRuntime.greedy_accept_commit(logits, mask, torch.from_numpy(verify).cuda(), start)
+        want = O.accept_commit(int(verify[0]), verify[1:], post, start)
+        np.testing.assert_array_equal(post_d.cpu().numpy().astype(np.uint32), post)
+        assert (res.acceptance_len, res.commit_count, res.staged_first_next, res.start) == (
+            want["acceptance_len"], want["commit_count"], want["staged_next"], want["start"])
+        assert res.acceptance_len == acc
+        start = res.start

@@ -451,3 +451,43 @@ def test_c_oracle_sdpa_and_accept():
     np.testing.assert_allclose(lse, lw, rtol=1e-5, atol=1e-5)
     assert c_oracle.match_acceptance_length([1, 2, 3], [1, 2, 5]) == 2
     assert c_oracle.match_acceptance_length([], []) == 0
+
+
+# ---- greedy tokens (DFlashRuntime.swift:105-128) ----
+
+def test_greedy_tokens_with_mask_brute_force():
+    rng = np.random.default_rng(3)
+    T, V = 5, 37
+    logits = rng.standard_normal((T, V)).astype(np.float32)
+    ids = [3, 36, -1, 99, 3]                                   # out-of-range ids are dropped (:109)
+    mask = O.build_suppress_token_mask(V, ids)
+    assert mask.sum() == 2 and mask[3] and mask[36]
+    assert O.build_suppress_token_mask(V, [-5, 400]) is None and O.build_suppress_token_mask(V, None) is None
+    got = O.greedy_tokens_with_mask(logits, mask)
+    for t in range(T):
+        best, arg = None, None
+        for v in range(V):
+            x = -1e9 if mask[v] else logits[t, v]
+            if best is None or x > best:
+                best, arg = x, v
+        assert got[t] == arg
+    assert got.dtype == np.uint32
+    # the row maximum sits on a suppressed token: the runner-up is returned
+    logits[0, 3] = 50.0
+    assert O.greedy_tokens_with_mask(logits, mask)[0] != 3
+    assert O.greedy_tokens_with_mask(logits, None)[0] == 3
+    # ties: lowest index
+    logits[1, :] = 0.0
+    assert O.greedy_tokens_with_mask(logits, None)[1] == 0
+
+
+def test_greedy_floor_is_rounded_to_the_logits_type():
+    """where(mask, MLXArray(-1e9, dtype: logits.dtype), logits): with every token suppressed the
+    floor ties everywhere and index 0 wins; a logit below the rounded floor loses to it."""
+    V = 8
+    mask = np.ones(V, bool)
+    assert O.greedy_tokens_with_mask(np.zeros((1, V), np.float32), mask, dtype="bf16")[0] == 0
+    mask[:] = False
+    mask[5] = True
+    low = np.full((1, V), -2e9, np.float32)
+    assert O.greedy_tokens_with_mask(low, mask, dtype="bf16")[0] == 5
