@@ -121,6 +121,60 @@ def cpu_baseline(stack_cfg, mean_commit: int):
     }
 
 
+def aux_kernels(lib, cfg, reps=48):
+    """The kernels on either side of the measured path, at the benchmark's shapes, each timed with
+    events attached to its dispatch over `reps` launches on rotating buffers (inputs come from HBM):
+    the GatedDelta pre-ops of one layer's 16-token block and the greedy tokens over [16, vocab]
+    logits fused with the acceptance bookkeeping.  Not part of `value`."""
+    import torch
+    from swiftlm_amd import DFlashKernels as K, DFlashRuntime as R, _lib
+
+    out = {}
+    dev, bf = "cuda", torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(11)
+    B, T, Hk, Hv, Dk, Dv, Kc = 1, cfg.block, cfg.Hk, cfg.Hv, cfg.Dk, cfg.Dv, 4
+    C = 2 * Hk * Dk + Hv * Dv
+    sets = [(torch.randn(B, T, C, generator=g, device=dev).to(bf), torch.randn(B, Kc - 1, C, generator=g, device=dev).to(bf),
+             torch.randn(B, T, Hv, generator=g, device=dev).to(bf), torch.randn(B, T, Hv, generator=g, device=dev).to(bf))
+            for _ in range(reps)]
+    w = (0.5 * torch.randn(C, Kc, generator=g, device=dev)).to(bf)
+    a_log = torch.randn(Hv, generator=g, device=dev)
+    dt_bias = torch.randn(Hv, generator=g, device=dev)
+    ev = HipEvents()
+    for x, st, a, b in sets[:4]:
+        K.gdn_prepare(x, st, w, a, b, a_log, dt_bias, Hk, Hv, Dk, Dv, 1.0 / Dk, Dk ** -0.5)
+    for x, st, a, b in sets:
+        e0, e1 = ev.pair()
+        _lib.check(lib.dflash_profile_next_launch(_lib.KERNEL_GDN_PREPARE, e0, e1), "profile_next_launch")
+        K.gdn_prepare(x, st, w, a, b, a_log, dt_bias, Hk, Hv, Dk, Dv, 1.0 / Dk, Dk ** -0.5)
+    torch.cuda.synchronize()
+    us = float(np.median(ev.durations_us()))
+    nbytes = (2 * T * C + 2 * (Kc - 1) * C + Kc * C + 4 * T * Hv) * 2        # x in/out, window in/out, taps, a/b/g/beta
+    out["gdn_prepare"] = {"us": round(us, 2), "algorithmic_bytes": nbytes, "gbs": round(nbytes / us / 1e3, 1),
+                          "shape": "B=1 T=%d C=%d K=%d bf16" % (T, C, Kc)}
+    ev.destroy()
+    del sets
+
+    V = 151936
+    logits = [torch.randn(T, V, generator=g, device=dev).to(bf) for _ in range(reps)]      # 48 x 4.9 MB
+    mask = R.build_suppress_token_mask(V, [1, 2, 3])
+    verify = torch.randint(0, V, (T,), generator=g, device=dev, dtype=torch.int32)
+    for lg in logits[:4]:
+        R.greedy_accept_commit(lg, mask, verify, 0)
+    ev = HipEvents()
+    for lg in logits:
+        e0, e1 = ev.pair()
+        _lib.check(lib.dflash_profile_next_launch(_lib.KERNEL_GREEDY_PARTIAL, e0, e1), "profile_next_launch")
+        R.greedy_accept_commit(lg, mask, verify, 0)
+    torch.cuda.synchronize()
+    us = float(np.median(ev.durations_us()))
+    nbytes = T * V * 2 + V
+    out["greedy_partial"] = {"us": round(us, 2), "algorithmic_bytes": nbytes, "gbs": round(nbytes / us / 1e3, 1),
+                             "shape": "T=%d V=%d bf16, uint8 suppress mask" % (T, V)}
+    ev.destroy()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -129,6 +183,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="enqueue every step from the host instead of replaying graphs")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--context", type=int, default=32768)
+    ap.add_argument("--aux", action="store_true",
+                    help="also time the kernels next to the measured path (pre-ops, greedy tokens) and report them "
+                         "under aux_kernels; they are not part of the step time")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy, the known-size kernel the rocprof byte counters are scaled by")
     args = ap.parse_args()
@@ -299,6 +356,8 @@ def main():
             "launches_timed": sdpa_launches,
         },
     }
+    if args.aux:
+        result["aux_kernels"] = aux_kernels(lib, cfg)
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
         dst = torch.empty_like(src)

@@ -120,6 +120,34 @@ int dflash_gated_delta_tape(void* stream,
                             int B, int T, int Hk, int Hv, int Dk, int Dv);
 
 /* ------------------------------------------------------------------------
+ * GatedDelta pre-ops: everything between the layer's projections and
+ * dflash_gated_delta_tape, in one launch (layer code around the recurrence,
+ * Sources/SwiftLM/KimiLinearDFlash.swift: ShortConv1d :274-293, q/k
+ * normalisation :362-363, gates :390-391).
+ *   mixed_qkv     [B, T, C], C = 2*Hk*Dk + Hv*Dv, channel order q | k | v
+ *   conv_state_in [B, K-1, C] or NULL (zeros, :288); conv_weight [C, K], tap j
+ *                 multiplies row t + j of concat(conv_state_in, mixed_qkv)
+ *   out = silu(conv)                                                    (:291)
+ *   q_out [B,T,Hk,Dk] = q_scale * rmsNorm(out_q, eps) per head; k_out likewise
+ *                 with k_scale (:362-363); v_out [B,T,Hv,Dv] = out_v
+ *   g_out = exp(-exp(A_log[h]) * softplus(a + dt_bias)), beta_out = sigmoid(b)
+ *                 (:390-391); g_ndim 3: a [B,T,Hv], dt_bias [Hv];
+ *                 g_ndim 4: a [B,T,Hv,Dk], dt_bias [Hv*Dk] (per-channel gate)
+ *   conv_state_out [B, K-1, C] = last K-1 rows of the concatenation (:292) --
+ *                 the window RecurrentRollbackCache snapshots; mixed_qkv itself is
+ *                 what recordTape keeps as qkv (RecurrentRollbackCache.swift:139-158).
+ * Tensors are `in_dtype` except A_log / dt_bias (float32 parameters).  2 <= K <= 8.
+ * ---------------------------------------------------------------------- */
+int dflash_gdn_prepare(void* stream,
+                       const void* mixed_qkv, const void* conv_state_in, const void* conv_weight,
+                       const void* a_logits, int g_ndim, const void* b_logits,
+                       const float* A_log, const float* dt_bias, int in_dtype,
+                       float q_scale, float k_scale, float norm_eps,
+                       void* q_out, void* k_out, void* v_out, void* g_out, void* beta_out,
+                       void* conv_state_out,
+                       int B, int T, int Hk, int Hv, int Dk, int Dv, int K);
+
+/* ------------------------------------------------------------------------
  * Block-causal batched GQA SDPA for the verify block.  Replaces
  * DFlashKernels.batchedSDPA2Pass (DFlashKernels.swift:737-815; Metal partials
  * :563-649, reduce :661-720); unlike it, covers every shape sdpaFallback
@@ -272,7 +300,8 @@ int dflash_kv_append(void* stream, void* k_cache, void* v_cache, const void* k_n
 #define DFLASH_KERNEL_GDN_FORWARD 2
 #define DFLASH_KERNEL_TAPE_REPLAY 3
 #define DFLASH_KERNEL_GREEDY_PARTIAL 4
-#define DFLASH_KERNEL_COUNT 5
+#define DFLASH_KERNEL_GDN_PREPARE 5
+#define DFLASH_KERNEL_COUNT 6
 int dflash_profile_next_launch(int kernel_id, void* start_event, void* stop_event);
 
 #ifdef __cplusplus

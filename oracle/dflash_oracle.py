@@ -184,6 +184,69 @@ def gated_delta_ops_with_tape(q, k, v, g, beta, state, mask=None, *, dtype=np.fl
 # ----------------------------------------------------------------------------
 
 
+# ---------------------------------------------------------------------------
+# GatedDelta pre-ops: short causal conv + SiLU, q/k normalisation, gate formulas
+# (the layer code around the recurrence: Sources/SwiftLM/KimiLinearDFlash.swift)
+# ---------------------------------------------------------------------------
+
+def short_conv_silu(x, conv_state, weight):
+    """``ShortConv1d`` (KimiLinearDFlash.swift:274-293): depthwise causal conv over
+    ``concat(state, x)`` along time, then SiLU.  x [B,T,C]; conv_state [B,K-1,C] or
+    None (zeros, :288); weight [C,K] (tap j multiplies the row j steps into the
+    window).  Returns (out [B,T,C], new_state [B,K-1,C] = the last K-1 rows of the
+    concatenation, :292)."""
+    x = np.asarray(x, dtype=np.float64)
+    w = np.asarray(weight, dtype=np.float64)
+    B, T, C = x.shape
+    K = w.shape[1]
+    prev = np.zeros((B, K - 1, C)) if conv_state is None else np.asarray(conv_state, dtype=np.float64)
+    ci = np.concatenate([prev, x], axis=1)                       # [B, T+K-1, C]
+    out = np.zeros((B, T, C))
+    for j in range(K):
+        out += ci[:, j:j + T, :] * w[None, None, :, j]
+    out = out / (1.0 + np.exp(-out))                             # silu (:291)
+    return out, ci[:, T:, :]
+
+
+def rms_norm_scaled(x, scale, eps=1e-6):
+    """``scale * rmsNorm(x, weight: none, eps)`` over the last axis (KimiLinearDFlash.swift:362-363)."""
+    x = np.asarray(x, dtype=np.float64)
+    return scale * x / np.sqrt((x * x).mean(axis=-1, keepdims=True) + eps)
+
+
+def gdn_gates(a_logits, b_logits, a_log, dt_bias):
+    """``g = exp(-exp(A_log) * softplus(a + dt_bias))``, ``beta = sigmoid(b)``
+    (KimiLinearDFlash.swift:390-391).  a_logits [B,T,H] with dt_bias [H], or
+    [B,T,H,Dk] with dt_bias [H,Dk]; a_log [H]."""
+    a = np.asarray(a_logits, dtype=np.float64)
+    al = np.asarray(a_log, dtype=np.float64)
+    db = np.asarray(dt_bias, dtype=np.float64)
+    if a.ndim == 4:
+        al = al[:, None]
+        db = db.reshape(a.shape[2], a.shape[3])
+    z = a + db
+    softplus = np.logaddexp(0.0, z)
+    g = np.exp(-np.exp(al) * softplus)
+    beta = 1.0 / (1.0 + np.exp(-np.asarray(b_logits, dtype=np.float64)))
+    return g, beta
+
+
+def gdn_prepare(mixed_qkv, conv_state, conv_weight, a_logits, b_logits, a_log, dt_bias,
+                Hk, Hv, Dk, Dv, q_scale, k_scale, eps=1e-6):
+    """The layer's steps between its projections and the recurrence
+    (KimiLinearDFlash.swift:351-364, :390-391) on the concatenated q|k|v channels:
+    conv+SiLU, split, ``q = q_scale * rmsNorm(q)``, ``k = k_scale * rmsNorm(k)`` per head,
+    gates.  Returns dict(q, k, v, g, beta, conv_state)."""
+    out, new_state = short_conv_silu(mixed_qkv, conv_state, conv_weight)
+    B, T, _ = out.shape
+    cq = Hk * Dk
+    q = rms_norm_scaled(out[..., :cq].reshape(B, T, Hk, Dk), q_scale, eps)
+    k = rms_norm_scaled(out[..., cq:2 * cq].reshape(B, T, Hk, Dk), k_scale, eps)
+    v = out[..., 2 * cq:].reshape(B, T, Hv, Dv)
+    g, beta = gdn_gates(a_logits, b_logits, a_log, dt_bias)
+    return dict(q=q, k=k, v=v, g=g, beta=beta, conv_state=new_state)
+
+
 def build_suppress_token_mask(vocab_size: int, suppress_token_ids):
     """Boolean [vocab] mask of the in-range ids, or None when there are none
     (DFlashRuntime.swift:105-115)."""

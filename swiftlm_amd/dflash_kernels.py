@@ -136,6 +136,42 @@ class DFlashKernels:
         return int(_lib.load().dflash_sdpa_workspace_bytes(B, Hq, Hk, M, N, D))
 
     @staticmethod
+    def gdn_prepare(mixed_qkv: torch.Tensor, conv_state: Optional[torch.Tensor], conv_weight: torch.Tensor,
+                    a_logits: torch.Tensor, b_logits: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
+                    Hk: int, Hv: int, Dk: int, Dv: int, q_scale: float, k_scale: float, eps: float = 1e-6):
+        """The layer's steps between its projections and the recurrence, in one launch
+        (Sources/SwiftLM/KimiLinearDFlash.swift: ShortConv1d :274-293, q/k normalisation :362-363,
+        gates :390-391).  ``mixed_qkv`` [B,T,2*Hk*Dk+Hv*Dv] with channels q|k|v; ``conv_state``
+        [B,K-1,C] or None; ``conv_weight`` [C,K]; ``a_logits`` [B,T,Hv] or [B,T,Hv,Dk];
+        ``a_log`` [Hv] and ``dt_bias`` float32.  Returns (q, k, v, g, beta, new_conv_state), ready for
+        ``gated_delta_kernel_with_tape``; ``mixed_qkv`` is what ``record_tape`` keeps as qkv."""
+        _dev(mixed_qkv, conv_state, conv_weight, a_logits, b_logits, a_log, dt_bias)
+        B, T, C = mixed_qkv.shape
+        if C != 2 * Hk * Dk + Hv * Dv:
+            raise DFlashError(f"gdn_prepare: {C} channels, expected 2*{Hk}*{Dk} + {Hv}*{Dv}")
+        K = int(conv_weight.shape[1])
+        dt = mixed_qkv.dtype
+        x = mixed_qkv.contiguous()
+        w = conv_weight.to(dt).contiguous()
+        st = None if conv_state is None else conv_state.to(dt).contiguous()
+        a = a_logits.to(dt).contiguous()
+        bl = b_logits.to(dt).contiguous()
+        al = a_log.float().contiguous()
+        db = dt_bias.float().contiguous().reshape(-1)
+        q = torch.empty(B, T, Hk, Dk, dtype=dt, device=x.device)
+        k = torch.empty_like(q)
+        v = torch.empty(B, T, Hv, Dv, dtype=dt, device=x.device)
+        g = torch.empty_like(a)
+        beta = torch.empty(B, T, Hv, dtype=dt, device=x.device)
+        new_state = torch.empty(B, K - 1, C, dtype=dt, device=x.device)
+        rc = _lib.load().dflash_gdn_prepare(
+            _stream(), _ptr(x), _ptr(st), _ptr(w), _ptr(a), a.dim(), _ptr(bl), _ptr(al), _ptr(db), _code(x),
+            float(q_scale), float(k_scale), float(eps), _ptr(q), _ptr(k), _ptr(v), _ptr(g), _ptr(beta), _ptr(new_state),
+            B, T, Hk, Hv, Dk, Dv, K)
+        _lib.check(rc, "gdn_prepare")
+        return q, k, v, g, beta, new_state
+
+    @staticmethod
     def batched_sdpa_2pass(queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, scale: float,
                            mask: Optional[torch.Tensor] = None, *, return_lse: bool = False,
                            kv_len: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None):

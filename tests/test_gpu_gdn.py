@@ -235,3 +235,81 @@ def test_unsupported_and_invalid_arguments(gpu_lib):
     with pytest.raises(DFlashError):                        # CPU tensors: there is no CPU path
         K.tape_replay_kernel(torch.zeros(1, 1, 4, 16), torch.zeros(1, 1, 2, 64), torch.zeros(1, 1, 4),
                              torch.zeros(1, 4, 16, 64))
+
+
+# ---- pre-ops: conv + SiLU, q/k normalisation, gates (KimiLinearDFlash.swift:274-293, :362-363, :390-391) ----
+
+def _prep_inputs(seed, B, T, Hk, Hv, Dk, Dv, K, vec):
+    rng = np.random.default_rng(seed)
+    C = 2 * Hk * Dk + Hv * Dv
+    return dict(
+        x=rng.standard_normal((B, T, C)).astype(np.float32),
+        state=rng.standard_normal((B, K - 1, C)).astype(np.float32),
+        w=(rng.standard_normal((C, K)) * 0.5).astype(np.float32),
+        a=(rng.standard_normal((B, T, Hv, Dk) if vec else (B, T, Hv)) * 2).astype(np.float32),
+        b=(rng.standard_normal((B, T, Hv)) * 2).astype(np.float32),
+        a_log=(rng.standard_normal(Hv) * 0.5).astype(np.float32),
+        dt_bias=rng.standard_normal((Hv, Dk) if vec else Hv).astype(np.float32),
+    )
+
+
+@pytest.mark.parametrize("cfg", [(1, 16, 16, 32, 128, 128, 4), (2, 5, 2, 4, 64, 96, 4), (1, 2, 1, 2, 32, 32, 4),
+                                 (1, 7, 2, 2, 128, 128, 2)],
+                         ids=["qwen3next_block", "ragged_dims", "T_shorter_than_window", "K2"])
+@pytest.mark.parametrize("vec", [False, True], ids=["scalar_g", "vec_g"])
+@pytest.mark.parametrize("in_dt", ["f32", "bf16"])
+def test_gdn_prepare_matches_oracle(gpu_lib, cfg, vec, in_dt):
+    from swiftlm_amd import DFlashKernels as K
+
+    B, T, Hk, Hv, Dk, Dv, Kc = cfg
+    if vec and Hk != Hv and False:
+        pytest.skip()
+    d = _prep_inputs(B * 100 + T, B, T, Hk, Hv, Dk, Dv, Kc, vec)
+    # the oracle sees exactly the values the device sees
+    rd = (lambda a: O.round_to_bf16(a)) if in_dt == "bf16" else (lambda a: a)
+    dd = {k: (rd(v) if k not in ("a_log", "dt_bias") else v) for k, v in d.items()}
+    want = O.gdn_prepare(dd["x"], dd["state"], dd["w"], dd["a"], dd["b"], dd["a_log"], dd["dt_bias"], Hk, Hv, Dk, Dv,
+                         q_scale=1.0 / Dk, k_scale=Dk ** -0.5)
+    got = K.gdn_prepare(dev(dd["x"], in_dt), dev(dd["state"], in_dt), dev(dd["w"], in_dt), dev(dd["a"], in_dt),
+                        dev(dd["b"], in_dt), dev(d["a_log"]), dev(d["dt_bias"]), Hk, Hv, Dk, Dv,
+                        q_scale=1.0 / Dk, k_scale=Dk ** -0.5)
+    torch.cuda.synchronize()
+    tol = dict(rtol=2e-5, atol=2e-6) if in_dt == "f32" else LOWP_TOL
+    for name, g in zip(("q", "k", "v", "g", "beta"), got[:5]):
+        np.testing.assert_allclose(host(g), want[name], err_msg=name, **tol)
+    np.testing.assert_array_equal(host(got[5]), want["conv_state"].astype(np.float32))      # copied rows: bit-exact
+    # no carried window = zeros
+    got0 = K.gdn_prepare(dev(dd["x"], in_dt), None, dev(dd["w"], in_dt), dev(dd["a"], in_dt), dev(dd["b"], in_dt),
+                         dev(d["a_log"]), dev(d["dt_bias"]), Hk, Hv, Dk, Dv, q_scale=1.0 / Dk, k_scale=Dk ** -0.5)
+    want0 = O.gdn_prepare(dd["x"], None, dd["w"], dd["a"], dd["b"], dd["a_log"], dd["dt_bias"], Hk, Hv, Dk, Dv,
+                          q_scale=1.0 / Dk, k_scale=Dk ** -0.5)
+    np.testing.assert_allclose(host(got0[2]), want0["v"], **tol)
+
+
+def test_gdn_prepare_feeds_the_forward_and_the_rollback_window(gpu_lib):
+    """pre-ops -> forward with tape -> conv-window rebuild after n accepted steps: the window equals
+    what the pre-ops leave after the first n tokens (RecurrentRollbackCache.swift:139-158)."""
+    from swiftlm_amd import DFlashKernels as K, _lib
+    from swiftlm_amd.dflash_kernels import _ptr, _stream
+
+    B, T, Hk, Hv, Dk, Dv, Kc = 1, 16, 4, 8, 128, 128, 4
+    d = _prep_inputs(9, B, T, Hk, Hv, Dk, Dv, Kc, False)
+    bf = lambda a: dev(O.round_to_bf16(a), "bf16")
+    x, st, w = bf(d["x"]), bf(d["state"]), bf(d["w"])
+    q, k, v, g, beta, new_state = K.gdn_prepare(x, st, w, bf(d["a"]), bf(d["b"]), dev(d["a_log"]), dev(d["dt_bias"]),
+                                                Hk, Hv, Dk, Dv, q_scale=1.0 / Dk, k_scale=Dk ** -0.5)
+    s0 = 0.1 * torch.randn(B, Hv, Dv, Dk, device="cuda")
+    y, s1, tape = K.gated_delta_kernel_with_tape(q, k, v, g, beta, s0)
+    yw, sw, tw = O.gated_delta_ops_with_tape(host(q), host(k), host(v), host(g), host(beta), host(s0))
+    np.testing.assert_allclose(host(s1), sw, **STATE_TOL)
+    np.testing.assert_allclose(host(y), yw, **LOWP_TOL)
+    lib = _lib.load()
+    C = x.shape[-1]
+    for n in (1, 5, 16):
+        out = torch.empty(B, Kc - 1, C, dtype=torch.bfloat16, device="cuda")
+        _lib.check(lib.dflash_rebuild_conv_state(_stream(), _ptr(st), _ptr(x), _ptr(out), B, Kc - 1, T, C, 2, n, None),
+                   "rebuild")
+        again = K.gdn_prepare(x[:, :n], st, w, bf(d["a"])[:, :n], bf(d["b"])[:, :n], dev(d["a_log"]), dev(d["dt_bias"]),
+                              Hk, Hv, Dk, Dv, q_scale=1.0 / Dk, k_scale=Dk ** -0.5)[5]
+        torch.cuda.synchronize()
+        assert torch.equal(out, again)

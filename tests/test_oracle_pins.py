@@ -491,3 +491,61 @@ def test_greedy_floor_is_rounded_to_the_logits_type():
     mask[5] = True
     low = np.full((1, V), -2e9, np.float32)
     assert O.greedy_tokens_with_mask(low, mask, dtype="bf16")[0] == 5
+
+
+# ---- GatedDelta pre-ops (KimiLinearDFlash.swift:274-293, :362-363, :390-391) ----
+
+def test_short_conv_is_a_causal_correlation_with_carried_window():
+    from scipy.signal import correlate
+    rng = np.random.default_rng(0)
+    B, T, C, K = 2, 9, 5, 4
+    x = rng.standard_normal((B, T, C))
+    st = rng.standard_normal((B, K - 1, C))
+    w = rng.standard_normal((C, K))
+    out, new = O.short_conv_silu(x, st, w)
+    for b in range(B):
+        for c in range(C):
+            full = np.concatenate([st[b, :, c], x[b, :, c]])
+            pre = correlate(full, w[c], mode="valid")                 # sum_j full[t+j] w[j]
+            np.testing.assert_allclose(out[b, :, c], pre / (1 + np.exp(-pre)), rtol=1e-12)
+    np.testing.assert_array_equal(new, np.concatenate([st, x], 1)[:, T:])
+    # processing the block in two pieces with the carried window equals one pass (what makes the
+    # window a sufficient state, and what rebuildConvState relies on)
+    o1, s1 = O.short_conv_silu(x[:, :4], st, w)
+    o2, s2 = O.short_conv_silu(x[:, 4:], s1, w)
+    np.testing.assert_allclose(np.concatenate([o1, o2], 1), out, rtol=1e-12)
+    np.testing.assert_array_equal(s2, new)
+    # no state = zeros (:288); T shorter than the window keeps old rows
+    o0, _ = O.short_conv_silu(x, None, w)
+    oz, _ = O.short_conv_silu(x, np.zeros_like(st), w)
+    np.testing.assert_array_equal(o0, oz)
+    _, s_short = O.short_conv_silu(x[:, :2], st, w)
+    np.testing.assert_array_equal(s_short, np.concatenate([st[:, 2:], x[:, :2]], 1))
+    # the rollback cache's rebuilt window after accepting n steps is the window a forward over the
+    # first n tokens would have left (RecurrentRollbackCache.swift:139-158)
+    for n in range(1, T + 1):
+        _, want = O.short_conv_silu(x[:, :n], st, w)
+        np.testing.assert_array_equal(O.rebuild_conv_state(st, x, n, K - 1), want)
+
+
+def test_rms_norm_and_gates_against_library_forms():
+    from scipy.special import expit
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((2, 3, 4, 16))
+    y = O.rms_norm_scaled(x, 16 ** -0.5, eps=0.0)
+    np.testing.assert_allclose(np.linalg.norm(y, axis=-1), 1.0, rtol=1e-12)      # scale * rmsNorm = L2 normalisation
+    a = rng.standard_normal((2, 3, 4)) * 3
+    b = rng.standard_normal((2, 3, 4)) * 3
+    al = rng.standard_normal(4)
+    db = rng.standard_normal(4)
+    g, beta = O.gdn_gates(a, b, al, db)
+    np.testing.assert_allclose(beta, expit(b), rtol=1e-12)
+    np.testing.assert_allclose(np.log(g), -np.exp(al) * np.log1p(np.exp(a + db)), rtol=1e-10)
+    assert np.all((g > 0) & (g <= 1))
+    # per-channel gate: each channel follows the scalar formula with its own bias
+    a4 = rng.standard_normal((1, 2, 4, 8))
+    db4 = rng.standard_normal((4, 8))
+    g4, _ = O.gdn_gates(a4, b[:1, :2], al, db4)
+    for d in range(8):
+        gd, _ = O.gdn_gates(a4[..., d], b[:1, :2], al, db4[:, d])
+        np.testing.assert_allclose(g4[..., d], gd, rtol=1e-12)
