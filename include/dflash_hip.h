@@ -147,6 +147,15 @@ int dflash_gdn_prepare(void* stream,
                        void* conv_state_out,
                        int B, int T, int Hk, int Hv, int Dk, int Dv, int K);
 
+/* The layer's step after the recurrence (KimiLinearDFlash.swift:377-378, RMSNorm :341):
+ *   out[b,t,h,:] = rmsNorm(y[b,t,h,:]; norm_weight [Dv], norm_eps) * act(gate[b,t,h,:])
+ * gate_kind 0: act = sigmoid (the in-tree layer); 1: act = silu (the gated RMSNorm of
+ * Qwen3-Next's linear-attention layer, whose source is not in the reference tree).
+ * y, gate, out [B,T,Hv,Dv] and norm_weight in `in_dtype`.
+ * ---------------------------------------------------------------------- */
+int dflash_gdn_finish(void* stream, const void* y, const void* gate, const void* norm_weight, void* out,
+                      int in_dtype, float norm_eps, int gate_kind, int B, int T, int Hv, int Dv);
+
 /* ------------------------------------------------------------------------
  * Block-causal batched GQA SDPA for the verify block.  Replaces
  * DFlashKernels.batchedSDPA2Pass (DFlashKernels.swift:737-815; Metal partials

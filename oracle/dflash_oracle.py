@@ -247,6 +247,16 @@ def gdn_prepare(mixed_qkv, conv_state, conv_weight, a_logits, b_logits, a_log, d
     return dict(q=q, k=k, v=v, g=g, beta=beta, conv_state=new_state)
 
 
+def gdn_finish(y, gate, norm_weight, eps, gate_kind="sigmoid"):
+    """``rmsNorm(y; weight, eps) * act(gate)`` over the last axis (KimiLinearDFlash.swift:377-378,
+    RMSNorm :341); act = sigmoid, or silu for the gated RMSNorm variant."""
+    y = np.asarray(y, dtype=np.float64)
+    z = np.asarray(gate, dtype=np.float64)
+    n = y / np.sqrt((y * y).mean(axis=-1, keepdims=True) + eps) * np.asarray(norm_weight, dtype=np.float64)
+    sig = 1.0 / (1.0 + np.exp(-z))
+    return n * (z * sig if gate_kind == "silu" else sig)
+
+
 def build_suppress_token_mask(vocab_size: int, suppress_token_ids):
     """Boolean [vocab] mask of the in-range ids, or None when there are none
     (DFlashRuntime.swift:105-115)."""

@@ -32,6 +32,7 @@ SIGNATURES = {
     "dflash_tape_replay_batched": (i32, [vp, i32, vpp, i32, vpp, vpp, i32, i32, vpp, vpp, i32, i32, vp, i32] + [i32] * 6),
     "dflash_gated_delta_tape": (i32, [vp, vp, vp, vp, vp, i32, vp, i32, vp, vp, i32, vp, vp, vp, i32] + [i32] * 6),
     "dflash_gdn_prepare": (i32, [vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, f32, f32, f32, vp, vp, vp, vp, vp, vp] + [i32] * 7),
+    "dflash_gdn_finish": (i32, [vp, vp, vp, vp, vp, i32, f32, i32, i32, i32, i32, i32]),
     "dflash_sdpa_workspace_bytes": (sz, [i32] * 6),
     "dflash_sdpa_block_causal": (i32, [vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp, vp, sz]),
     "dflash_sdpa_block_causal_masked": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp, vp, sz]),

@@ -124,9 +124,75 @@ __global__ void gdn_prepare_kernel(PrepareArgs A) {
     }
 }
 
+// ---- post-op: out = rmsNorm(y; weight, eps) * act(gate) per head --------------------------
+// (KimiLinearDFlash.swift:377-378: oNorm(out) * sigmoid(gate); RMSNorm with a learned weight of
+// headDim elements, :341.)  One wave per (b, t, head) row of Dv elements.
+struct FinishArgs {
+    const void* y;        // [rows, Dv]
+    const void* gate;     // [rows, Dv]
+    const void* weight;   // [Dv]
+    void* out;            // [rows, Dv]
+    float eps;
+    int rows, Dv, silu_gate;
+};
+
+template <typename Elem>
+__global__ __launch_bounds__(256) void gdn_finish_kernel(FinishArgs A) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= A.rows) return;
+    const Elem* y = reinterpret_cast<const Elem*>(A.y) + (size_t)row * A.Dv;
+    const Elem* gt = reinterpret_cast<const Elem*>(A.gate) + (size_t)row * A.Dv;
+    const Elem* wt = reinterpret_cast<const Elem*>(A.weight);
+    Elem* out = reinterpret_cast<Elem*>(A.out) + (size_t)row * A.Dv;
+    constexpr int kMaxPer = 16;                      // Dv <= 1024
+    float v[kMaxPer];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxPer; ++i) {
+        const int d = lane + 64 * i;
+        v[i] = d < A.Dv ? to_float(y[d]) : 0.f;
+        ss = fmaf(v[i], v[i], ss);
+    }
+    for (int o = 32; o >= 1; o >>= 1) ss += __shfl_xor(ss, o);
+    const float inv = rsqrtf(ss / (float)A.Dv + A.eps);
+#pragma unroll
+    for (int i = 0; i < kMaxPer; ++i) {
+        const int d = lane + 64 * i;
+        if (d < A.Dv) {
+            const float z = to_float(gt[d]);
+            const float act = A.silu_gate ? z * sigmoid_f(z) : sigmoid_f(z);
+            out[d] = from_float<Elem>(v[i] * inv * to_float(wt[d]) * act);
+        }
+    }
+}
+
 }  // namespace dflash
 
 using namespace dflash;
+
+extern "C" int dflash_gdn_finish(void* stream, const void* y, const void* gate, const void* norm_weight, void* out,
+                                 int in_dtype, float norm_eps, int gate_kind, int B, int T, int Hv, int Dv) {
+    int rc = ensure_init();
+    if (rc) return rc;
+    DFLASH_REQUIRE(y && gate && norm_weight && out, "gdn_finish: null pointer");
+    DFLASH_REQUIRE(B > 0 && T > 0 && Hv > 0 && Dv > 0, "gdn_finish: non-positive dimension");
+    DFLASH_REQUIRE(gate_kind == 0 || gate_kind == 1, "gdn_finish: gate_kind must be 0 (sigmoid) or 1 (silu)");
+    DFLASH_SUPPORTED(Dv <= 1024, "gdn_finish: head dim above 1024");
+    DFLASH_SUPPORTED(in_dtype == DFLASH_F32 || in_dtype == DFLASH_BF16 || in_dtype == DFLASH_F16, "gdn_finish: bad dtype %d", in_dtype);
+    const long rows = (long)B * T * Hv;
+    DFLASH_REQUIRE(rows <= 0x7fffffffL, "gdn_finish: too many rows");
+    FinishArgs A;
+    A.y = y; A.gate = gate; A.weight = norm_weight; A.out = out; A.eps = norm_eps;
+    A.rows = (int)rows; A.Dv = Dv; A.silu_gate = gate_kind;
+    dim3 grid((unsigned)((rows + 3) / 4));
+    hipStream_t st = (hipStream_t)stream;
+    if (in_dtype == DFLASH_F32) hipLaunchKernelGGL(gdn_finish_kernel<float>, grid, dim3(256), 0, st, A);
+    else if (in_dtype == DFLASH_BF16) hipLaunchKernelGGL(gdn_finish_kernel<bf16_t>, grid, dim3(256), 0, st, A);
+    else hipLaunchKernelGGL(gdn_finish_kernel<f16_t>, grid, dim3(256), 0, st, A);
+    DFLASH_HIP_TRY(hipGetLastError());
+    return DFLASH_OK;
+}
 
 extern "C" int dflash_gdn_prepare(void* stream, const void* mixed_qkv, const void* conv_state_in,
                                   const void* conv_weight, const void* a_logits, int g_ndim, const void* b_logits,

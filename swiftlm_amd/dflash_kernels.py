@@ -172,6 +172,23 @@ class DFlashKernels:
         return q, k, v, g, beta, new_state
 
     @staticmethod
+    def gdn_finish(y: torch.Tensor, gate: torch.Tensor, norm_weight: torch.Tensor, eps: float,
+                   gate_kind: str = "sigmoid") -> torch.Tensor:
+        """``oNorm(out) * sigmoid(gate)`` per head (KimiLinearDFlash.swift:377-378); ``gate_kind="silu"``
+        is the gated RMSNorm of Qwen3-Next's layer.  y, gate [B,T,Hv,Dv]; norm_weight [Dv]."""
+        _dev(y, gate, norm_weight)
+        if y.dim() != 4 or gate.shape != y.shape or norm_weight.shape != (y.shape[3],):
+            raise DFlashError("gdn_finish: y and gate must be [B,T,Hv,Dv], norm_weight [Dv]")
+        B, T, Hv, Dv = y.shape
+        y = y.contiguous()
+        out = torch.empty_like(y)
+        rc = _lib.load().dflash_gdn_finish(_stream(), _ptr(y), _ptr(gate.to(y.dtype).contiguous()),
+                                           _ptr(norm_weight.to(y.dtype).contiguous()), _ptr(out), _code(y), float(eps),
+                                           {"sigmoid": 0, "silu": 1}[gate_kind], B, T, Hv, Dv)
+        _lib.check(rc, "gdn_finish")
+        return out
+
+    @staticmethod
     def batched_sdpa_2pass(queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, scale: float,
                            mask: Optional[torch.Tensor] = None, *, return_lse: bool = False,
                            kv_len: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None):

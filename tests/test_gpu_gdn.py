@@ -313,3 +313,20 @@ def test_gdn_prepare_feeds_the_forward_and_the_rollback_window(gpu_lib):
                               Hk, Hv, Dk, Dv, q_scale=1.0 / Dk, k_scale=Dk ** -0.5)[5]
         torch.cuda.synchronize()
         assert torch.equal(out, again)
+
+
+@pytest.mark.parametrize("kind", ["sigmoid", "silu"])
+@pytest.mark.parametrize("in_dt", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("shape", [(1, 16, 32, 128), (2, 3, 5, 40), (1, 2, 2, 200)], ids=["block", "odd", "wide"])
+def test_gdn_finish_matches_oracle(gpu_lib, shape, in_dt, kind):
+    from swiftlm_amd import DFlashKernels as K
+
+    rng = np.random.default_rng(sum(shape))
+    rd = {"f32": lambda a: a, "bf16": O.round_to_bf16, "f16": lambda a: a.astype(np.float16).astype(np.float32)}[in_dt]
+    y = rd(rng.standard_normal(shape).astype(np.float32))
+    z = rd((rng.standard_normal(shape) * 2).astype(np.float32))
+    w = rd((1 + 0.1 * rng.standard_normal(shape[-1])).astype(np.float32))
+    got = K.gdn_finish(dev(y, in_dt), dev(z, in_dt), dev(w, in_dt), 1e-6, kind)
+    torch.cuda.synchronize()
+    tol = dict(rtol=2e-5, atol=2e-6) if in_dt == "f32" else LOWP_TOL
+    np.testing.assert_allclose(host(got), O.gdn_finish(y, z, w, 1e-6, kind), **tol)

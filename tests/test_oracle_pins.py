@@ -549,3 +549,17 @@ def test_rms_norm_and_gates_against_library_forms():
     for d in range(8):
         gd, _ = O.gdn_gates(a4[..., d], b[:1, :2], al, db4[:, d])
         np.testing.assert_allclose(g4[..., d], gd, rtol=1e-12)
+
+
+def test_gdn_finish_against_library_forms():
+    from scipy.special import expit
+    rng = np.random.default_rng(2)
+    y = rng.standard_normal((2, 3, 4, 16))
+    z = rng.standard_normal((2, 3, 4, 16)) * 3
+    w = rng.standard_normal(16)
+    out = O.gdn_finish(y, z, w, 0.0)
+    # with eps = 0 and unit weight the normalised rows have RMS 1; undo the gate to see it
+    unit = O.gdn_finish(y, z, np.ones(16), 0.0) / expit(z)
+    np.testing.assert_allclose(np.sqrt((unit ** 2).mean(-1)), 1.0, rtol=1e-12)
+    np.testing.assert_allclose(out, unit * w * expit(z), rtol=1e-12)
+    np.testing.assert_allclose(O.gdn_finish(y, z, w, 1e-6, "silu"), O.gdn_finish(y, z, w, 1e-6) * z, rtol=1e-12)
