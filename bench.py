@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """DFlash verify-step benchmark on one MI355X.
 
-A "step" is one verify step of the hybrid stack of BASELINE config 4: 48 layers =
+A "step" is one verify step of the hybrid stack of the headline benchmark configuration: 48 layers =
 12 x (GatedDelta, GatedDelta, GatedDelta, attention), 16-token draft block, 32K
 context, accepted length ~ Geometric(0.25) clipped to [1, 16].  Per step: 36
 GatedDelta forwards with tape, 12 KV appends + block-causal SDPAs, the accept kernel

@@ -517,7 +517,7 @@ def sdpa_2pass(q, k, v, scale, blocks=32, *, partial_dtype="bf16"):
 
 
 # ----------------------------------------------------------------------------
-# synthetic inputs of the BASELINE configs
+# synthetic inputs of the benchmark configurations
 # ----------------------------------------------------------------------------
 
 
@@ -544,7 +544,7 @@ def make_gdn_inputs(seed, B, T, Hk, Hv, Dk, Dv, *, in_dtype="f32", vec_gate=Fals
 
 
 def draw_accepted(rng, T, kind="uniform"):
-    """BASELINE's accepted length n in [1, T]: uniform (config 0) or Geometric(0.25) clipped."""
+    """The benchmark's accepted length n in [1, T]: uniform (config 0) or Geometric(0.25) clipped."""
     if kind == "uniform":
         return int(rng.integers(1, T + 1))
     return int(min(rng.geometric(0.25), T))

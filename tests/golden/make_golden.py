@@ -59,7 +59,7 @@ def accept_fixture(name, seed, n_cases=64):
 
 
 if __name__ == "__main__":
-    # BASELINE config 0 (fp32, the reference's CPU-runnable case), n ~ U{1..8} drawn with the seed
+    # benchmark configuration 0 (fp32, the reference's CPU-runnable case), n ~ U{1..8} drawn with the seed
     gdn_fixture("gdn_config0_f32.npz", 0, 1, 8, 4, 8, 64, 64, "f32", False, False,
                 O.draw_accepted(np.random.default_rng(0), 8, "uniform"))
     # a slice of the Qwen3-Next shape (4 of 32 value heads), bf16 inputs, n ~ Geometric(0.25)

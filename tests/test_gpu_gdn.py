@@ -1,7 +1,7 @@
 """GPU parity: GatedDelta forward-with-tape and tape replay (HIP, through the C ABI)
 against the CPU oracle on the same seeded inputs.
 
-Bars (BASELINE north_star): fp32 recurrent state rtol 1e-4 (atol 1e-6 for entries
+Bars: fp32 recurrent state rtol 1e-4 (atol 1e-6 for entries
 near zero); bf16/f16 outputs 2e-2 abs/rel; the fp32 tape is held to the state's bar.
 """
 

@@ -2,7 +2,7 @@
 CPU oracle, and at the long-context sizes against size-independent properties and
 a float32 torch restatement of the same op.
 
-Bar (BASELINE north_star): bf16/f16 outputs within 2e-2 abs/rel; the float32
+Bar: bf16/f16 outputs within 2e-2 abs/rel; the float32
 logsumexp is held to 2e-3 (its inputs are bf16 products accumulated in fp32)."""
 
 import math
@@ -79,7 +79,7 @@ def test_sdpa_matches_oracle_small(gpu_lib, cfg, dtype):
 
 
 def test_sdpa_config2_against_c_oracle(gpu_lib):
-    """BASELINE config 2: Hq=16, Hkv=2, D=256, L=4096, scale 1/16."""
+    """Benchmark configuration 2: Hq=16, Hkv=2, D=256, L=4096, scale 1/16."""
     from swiftlm_amd import DFlashKernels as K
 
     q, k, v = gpu_inputs(2, 1, 16, 2, 4096, 256)
@@ -100,7 +100,7 @@ def test_sdpa_config2_against_c_oracle(gpu_lib):
 
 @pytest.mark.parametrize("L", [32768, 40960, 102400])
 def test_sdpa_long_context_properties(gpu_lib, L):
-    """BASELINE config 3 sizes.  Properties that do not need a CPU pass: constant V gives
+    """Benchmark configuration 3 sizes.  Properties that do not need a CPU pass: constant V gives
     constant O; the result matches a float32 restatement; appending hidden (future) keys
     changes nothing for the rows that cannot see them."""
     from swiftlm_amd import DFlashKernels as K
@@ -121,7 +121,7 @@ def test_sdpa_long_context_properties(gpu_lib, L):
 
 
 def test_sdpa_ragged_batch(gpu_lib):
-    """BASELINE config 3's ragged batch: 4 sequences with L ~ U[8K, 64K], one launch,
+    """Benchmark configuration 3's ragged batch: 4 sequences with L ~ U[8K, 64K], one launch,
     per-sequence key counts on the device."""
     from swiftlm_amd import DFlashKernels as K
 
