@@ -272,3 +272,15 @@ def test_greedy_accept_commit_equals_two_steps(gpu_lib):
             want["acceptance_len"], want["commit_count"], want["staged_next"], want["start"])
         assert res.acceptance_len == acc
         start = res.start
+
+
+def test_plain_c_client_of_the_abi(gpu_lib):
+    """tests/cabi_c/cabi_check.c, built with gcc as C99 against include/dflash_hip.h: tape replay against
+    the recurrence computed on the host in C, the acceptance bookkeeping, and an unsupported shape."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "swiftlm_amd", "lib", "cabi_check")
+    assert os.path.exists(exe), "build it with `make -C swiftlm_amd/csrc`"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "C ABI check passed" in r.stdout
