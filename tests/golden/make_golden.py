@@ -58,6 +58,47 @@ def accept_fixture(name, seed, n_cases=64):
     np.savez_compressed(os.path.join(HERE, name), cases=np.array(rows, dtype=np.int64))
 
 
+def preops_fixture(name, seed, B, T, Hk, Hv, Dk, Dv, K):
+    """bf16-representable inputs of the GatedDelta pre/post-ops and their float64 results."""
+    rng = np.random.default_rng(seed)
+    C = 2 * Hk * Dk + Hv * Dv
+    r = lambda a: O.round_to_bf16(a.astype(np.float32))
+    d = dict(x=r(rng.standard_normal((B, T, C))), conv_state=r(rng.standard_normal((B, K - 1, C))),
+             conv_weight=r(0.5 * rng.standard_normal((C, K))), a=r(2 * rng.standard_normal((B, T, Hv))),
+             b=r(2 * rng.standard_normal((B, T, Hv))), a_log=(0.5 * rng.standard_normal(Hv)).astype(np.float32),
+             dt_bias=rng.standard_normal(Hv).astype(np.float32), gate=r(2 * rng.standard_normal((B, T, Hv, Dv))),
+             norm_weight=r(1 + 0.1 * rng.standard_normal(Dv)))
+    o = O.gdn_prepare(d["x"], d["conv_state"], d["conv_weight"], d["a"], d["b"], d["a_log"], d["dt_bias"], Hk, Hv, Dk, Dv,
+                      q_scale=1.0 / Dk, k_scale=Dk ** -0.5)
+    fin = O.gdn_finish(o["v"], d["gate"], d["norm_weight"], 1e-6)        # the post-op applied to v as a stand-in for y
+    np.savez_compressed(os.path.join(HERE, name), dims=np.array([B, T, Hk, Hv, Dk, Dv, K]), **d,
+                        **{"out_" + k: v.astype(np.float32) for k, v in o.items()}, out_finish=fin.astype(np.float32))
+
+
+def greedy_fixture(name, seed, T, V):
+    rng = np.random.default_rng(seed)
+    logits = O.round_to_bf16((4 * rng.standard_normal((T, V))).astype(np.float32))
+    ids = [0, 7, V - 1, V + 5] + list(range(100, 140))
+    logits[0, 7] = 64.0                 # the unmasked winner is suppressed
+    logits[1, 50] = logits[1, 900] = 63.0   # a tie: the lower index wins
+    mask = O.build_suppress_token_mask(V, ids)
+    np.savez_compressed(os.path.join(HERE, name), logits=logits, suppress_ids=np.array(ids),
+                        tokens_masked=O.greedy_tokens_with_mask(logits, mask, dtype="bf16"),
+                        tokens_plain=O.greedy_tokens_with_mask(logits, None, dtype="bf16"))
+
+
+def sdpa_masked_fixture(name, seed, B, Hq, Hk, L, D, scale):
+    q, k, v = O.make_sdpa_inputs(seed, B, Hq, Hk, 16, L, D)
+    rng = np.random.default_rng(seed + 1)
+    N = L + 16
+    mask = O.round_to_bf16(rng.standard_normal((B, Hq, 16, N)).astype(np.float32))
+    mask[rng.random((B, Hq, 16, N)) < 0.25] = -np.inf
+    mask[0, 0, 3, :] = -np.inf          # a row without usable keys: zeros
+    o, lse = O.sdpa_block_causal(q, k, v, scale, mask.astype(np.float64))
+    np.savez_compressed(os.path.join(HERE, name), q=q, k=k, v=v, mask=mask, scale=scale, out=o.astype(np.float32),
+                        lse=lse.astype(np.float32))
+
+
 if __name__ == "__main__":
     # benchmark configuration 0 (fp32, the reference's CPU-runnable case), n ~ U{1..8} drawn with the seed
     gdn_fixture("gdn_config0_f32.npz", 0, 1, 8, 4, 8, 64, 64, "f32", False, False,
@@ -69,4 +110,7 @@ if __name__ == "__main__":
     sdpa_fixture("sdpa_small_d256.npz", 3, 1, 16, 2, 200, 256, 1.0 / 16)
     sdpa_fixture("sdpa_small_d128.npz", 4, 2, 8, 2, 77, 128, 1.0 / np.sqrt(128))
     accept_fixture("accept_commit_cases.npz", 5)
+    preops_fixture("preops_gdn_bf16.npz", 6, 1, 6, 2, 4, 64, 64, 4)
+    greedy_fixture("greedy_tokens_bf16.npz", 7, 16, 5000)
+    sdpa_masked_fixture("masked_sdpa_d128.npz", 8, 1, 4, 2, 60, 128, 1.0 / np.sqrt(128))
     print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith(".npz")))

@@ -118,3 +118,57 @@ def test_hip_matches_accept_fixture(gpu_lib):
     for row in load("accept_commit_cases.npz")["cases"]:
         r = R.accept_commit(torch.from_numpy(row[0:16]).cuda(), torch.from_numpy(row[16:32]).cuda(), int(row[32]))
         assert [r.acceptance_len, r.commit_count, r.staged_first_next, r.start] == list(row[33:37])
+
+
+# ---- fixtures of the ops next to the verify path ----
+
+def test_oracles_reproduce_new_fixtures():
+    f = load("preops_gdn_bf16.npz")
+    B, T, Hk, Hv, Dk, Dv, K = [int(x) for x in f["dims"]]
+    o = O.gdn_prepare(f["x"], f["conv_state"], f["conv_weight"], f["a"], f["b"], f["a_log"], f["dt_bias"], Hk, Hv, Dk, Dv,
+                      q_scale=1.0 / Dk, k_scale=Dk ** -0.5)
+    for k, v in o.items():
+        np.testing.assert_allclose(v, f["out_" + k], rtol=1e-6, atol=1e-7, err_msg=k)
+    np.testing.assert_allclose(O.gdn_finish(o["v"], f["gate"], f["norm_weight"], 1e-6), f["out_finish"], rtol=1e-6, atol=1e-7)
+    g = load("greedy_tokens_bf16.npz")
+    mask = O.build_suppress_token_mask(g["logits"].shape[1], g["suppress_ids"].tolist())
+    np.testing.assert_array_equal(O.greedy_tokens_with_mask(g["logits"], mask, dtype="bf16"), g["tokens_masked"])
+    np.testing.assert_array_equal(O.greedy_tokens_with_mask(g["logits"], None, dtype="bf16"), g["tokens_plain"])
+    assert g["tokens_masked"][0] != 7 and g["tokens_plain"][0] == 7 and g["tokens_plain"][1] == 50
+    m = load("masked_sdpa_d128.npz")
+    o2, lse = O.sdpa_block_causal(m["q"], m["k"], m["v"], float(m["scale"]), m["mask"].astype(np.float64))
+    np.testing.assert_allclose(o2, m["out"], rtol=1e-5, atol=1e-6)
+    assert np.all(m["out"][0, 0, 3] == 0) and m["lse"][0, 0, 3] == -np.inf
+
+
+@pytest.mark.gpu
+def test_hip_matches_new_fixtures(gpu_lib):
+    import torch
+
+    from swiftlm_amd import DFlashKernels as K, DFlashRuntime as R
+
+    bf = torch.bfloat16
+    f = load("preops_gdn_bf16.npz")
+    B, T, Hk, Hv, Dk, Dv, Kc = [int(x) for x in f["dims"]]
+    got = K.gdn_prepare(_dev(f["x"], bf), _dev(f["conv_state"], bf), _dev(f["conv_weight"], bf), _dev(f["a"], bf),
+                        _dev(f["b"], bf), _dev(f["a_log"], torch.float32), _dev(f["dt_bias"], torch.float32),
+                        Hk, Hv, Dk, Dv, q_scale=1.0 / Dk, k_scale=Dk ** -0.5)
+    for name, t in zip(("q", "k", "v", "g", "beta"), got[:5]):
+        np.testing.assert_allclose(t.float().cpu().numpy(), f["out_" + name], rtol=2e-2, atol=2e-2, err_msg=name)
+    np.testing.assert_array_equal(got[5].float().cpu().numpy(), f["out_conv_state"])
+    fin = K.gdn_finish(_dev(f["out_v"], bf), _dev(f["gate"], bf), _dev(f["norm_weight"], bf), 1e-6)
+    np.testing.assert_allclose(fin.float().cpu().numpy(),
+                               O.gdn_finish(O.round_to_bf16(f["out_v"]), f["gate"], f["norm_weight"], 1e-6), rtol=2e-2, atol=2e-2)
+    g = load("greedy_tokens_bf16.npz")
+    V = g["logits"].shape[1]
+    mask = R.build_suppress_token_mask(V, g["suppress_ids"].tolist())
+    lg = _dev(g["logits"], bf)
+    np.testing.assert_array_equal(R.greedy_tokens_with_mask(lg, mask).cpu().numpy().astype(np.uint32), g["tokens_masked"])
+    np.testing.assert_array_equal(R.greedy_tokens_with_mask(lg, None).cpu().numpy().astype(np.uint32), g["tokens_plain"])
+    m = load("masked_sdpa_d128.npz")
+    out, lse = K.batched_sdpa_2pass(_dev(m["q"], bf), _dev(m["k"], bf), _dev(m["v"], bf), float(m["scale"]),
+                                    _dev(m["mask"], bf), return_lse=True)
+    np.testing.assert_allclose(out.float().cpu().numpy(), m["out"], rtol=2e-2, atol=2e-2)
+    fin_rows = np.isfinite(m["lse"])
+    np.testing.assert_allclose(lse.cpu().numpy()[fin_rows], m["lse"][fin_rows], rtol=2e-3, atol=2e-3)
+    assert lse.cpu().numpy()[0, 0, 3] == -np.inf
