@@ -241,6 +241,19 @@ int dflash_match_acceptance_length(void* stream, const uint32_t* drafted, const 
 int dflash_accept_commit(void* stream, const uint32_t* verify_ids, const uint32_t* posterior, int V,
                          int32_t* start_inout, int32_t* out4);
 
+/* dflash_accept_commit and dflash_tape_replay_batched in ONE launch: the replay kernel
+ * decides the acceptance itself (steps = commitCount = 1 + acceptanceLen; with
+ * skip_if_full a fully accepted block, commitCount == T_tape, writes no state) and
+ * leaves out4 / start_inout exactly as dflash_accept_commit would.  V <= T_tape + 1.
+ * Arguments as for the two calls it replaces (DFlashRuntime.swift:525-547 followed
+ * by the per-cache loop :197-205). */
+int dflash_accept_commit_replay_batched(void* stream, const uint32_t* verify_ids, const uint32_t* posterior,
+                                        int V, int32_t* start_inout, int32_t* out4, int n_layers,
+                                        const void* const* tape, int tape_dtype, const void* const* k,
+                                        const void* const* g, int in_dtype, int g_ndim,
+                                        const void* const* state_in, void* const* state_out, int state_dtype,
+                                        int skip_if_full, int B, int T_tape, int Hk, int Hv, int Dk, int Dv);
+
 /* ------------------------------------------------------------------------
  * Greedy tokens over the verify logits.  dflash_greedy_tokens_with_mask replaces
  * DFlashRuntime.greedyTokensWithMask (DFlashRuntime.swift:118-128):

@@ -134,6 +134,21 @@ __device__ __forceinline__ bool mask_on(const void* mask, int mask_dtype, int id
 // ---- cross-lane sums inside one 16-lane DPP row ---------------------------
 // Data-parallel-primitive controls of GFX9: quad_perm, row_half_mirror, row_mirror.
 
+// One wave.  Leading-match count = index of the first mismatch (n if none);
+// equals sum(cumprod(drafted == posterior)) (DFlashRuntime.swift:139-141).
+__device__ __forceinline__ int leading_matches(const uint32_t* a, const uint32_t* b, int n) {
+    const int lane = threadIdx.x;
+    int first = n;
+    for (int base = 0; base < n; base += 64) {
+        const int i = base + lane;
+        const bool mismatch = i < n && a[i] != b[i];
+        const unsigned long long bal = __builtin_amdgcn_ballot_w64(mismatch);
+        if (bal) { first = base + __builtin_ctzll(bal); break; }   // uniform
+    }
+    return first;
+}
+
+
 template <int CTRL> __device__ __forceinline__ float dpp_add(float x) {
     int y = __builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false);
     return x + __int_as_float(y);

@@ -63,20 +63,6 @@ LaunchBracket::LaunchBracket(int kernel_id, hipStream_t st) : stream(st), start(
 
 // ---- acceptance ------------------------------------------------------------
 
-// One wave.  Leading-match count = index of the first mismatch (n if none);
-// equals sum(cumprod(drafted == posterior)) (DFlashRuntime.swift:139-141).
-__device__ __forceinline__ int leading_matches(const uint32_t* a, const uint32_t* b, int n) {
-    const int lane = threadIdx.x;
-    int first = n;
-    for (int base = 0; base < n; base += 64) {
-        const int i = base + lane;
-        const bool mismatch = i < n && a[i] != b[i];
-        const unsigned long long bal = __builtin_amdgcn_ballot_w64(mismatch);
-        if (bal) { first = base + __builtin_ctzll(bal); break; }   // uniform
-    }
-    return first;
-}
-
 __global__ __launch_bounds__(64) void match_acceptance_kernel(const uint32_t* drafted, const uint32_t* posterior,
                                                               int n, int32_t* out) {
     const int acc = leading_matches(drafted, posterior, n);
@@ -376,6 +362,12 @@ extern "C" int dflash_rebuild_conv_state(void* stream, const void* snapshot_conv
     DFLASH_REQUIRE(((long)C * elem_bytes) % 16 == 0, "rebuild_conv_state: row of %d x %d bytes is not a multiple of 16", C, elem_bytes);
     DFLASH_REQUIRE(((uintptr_t)snapshot_conv | (uintptr_t)tape_qkv | (uintptr_t)out) % 16 == 0, "rebuild_conv_state: pointers must be 16-byte aligned");
     DFLASH_REQUIRE(keep <= 65535 && B <= 65535, "rebuild_conv_state: keep or B too large");
+    {
+        const size_t win = (size_t)B * keep * C * elem_bytes, tape_bytes = (size_t)B * T * C * elem_bytes;
+        const uintptr_t o = (uintptr_t)out, q = (uintptr_t)tape_qkv, sn = (uintptr_t)snapshot_conv;
+        DFLASH_REQUIRE(!(o < q + tape_bytes && q < o + win) && !(sn && o < sn + win && sn < o + win),
+                       "rebuild_conv_state: out overlaps an input");
+    }
     const int C16 = (int)(((long)C * elem_bytes) / 16);
     dim3 grid((C16 + 255) / 256, keep, B);
     hipLaunchKernelGGL(rebuild_conv_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const uint4*)snapshot_conv,

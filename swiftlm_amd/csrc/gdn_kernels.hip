@@ -56,6 +56,12 @@ struct ReplayBatch {
 struct ReplayArgs {
     const void* mask;        // [B,T_tape] or null
     const int32_t* steps_dev;
+    // fused acceptance (null verify_ids = off): steps = 1 + leading matches of verify_ids[1:] vs posterior
+    const uint32_t* verify_ids;
+    const uint32_t* posterior;
+    int32_t* start_inout;
+    int32_t* out4;
+    int V;
     int mask_dtype, tape_dtype, in_dtype;
     int steps, skip_if_full;
     int T_tape, Hk, Hv, Dv;
@@ -89,7 +95,31 @@ __global__ __launch_bounds__(kThreads) void tape_replay_kernel(ReplayBatch P, Re
     const bool owner = tid < RPP * TPR;            // false only for the spare threads of an odd TPR
     const int rsub = owner ? tid / TPR : 0;
 
-    int n = A.steps_dev ? *A.steps_dev : A.steps;
+    int n;
+    if (A.verify_ids) {
+        // The cycle's acceptance (DFlashRuntime.swift:525-547) is decided here, by every workgroup for
+        // itself (two 64-byte reads), so the rollback needs no launch ahead of it; workgroup 0 also does
+        // the bookkeeping accept_commit_kernel would have done.
+        __shared__ int n_s;
+        if (tid < 64) {
+            const int acc = A.V > 1 ? leading_matches(A.verify_ids + 1, A.posterior, A.V - 1) : 0;
+            if (tid == 0) {
+                n_s = 1 + acc;
+                if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0) {
+                    A.out4[0] = acc;
+                    A.out4[1] = 1 + acc;
+                    A.out4[2] = (int32_t)A.posterior[acc];
+                    int start = 1 + acc;
+                    if (A.start_inout) { start += *A.start_inout; *A.start_inout = start; }
+                    A.out4[3] = start;
+                }
+            }
+        }
+        __syncthreads();
+        n = n_s;
+    } else {
+        n = A.steps_dev ? *A.steps_dev : A.steps;
+    }
     n = n < 0 ? 0 : (n > A.T_tape ? A.T_tape : n);
     if (A.skip_if_full && n == A.T_tape) return;   // uniform over the grid
 
@@ -196,11 +226,19 @@ static int launch_replay_state(hipStream_t st, const ReplayBatch& P, const Repla
     return DFLASH_UNSUPPORTED;
 }
 
+struct FusedAccept {
+    const uint32_t* verify_ids = nullptr;
+    const uint32_t* posterior = nullptr;
+    int32_t* start_inout = nullptr;
+    int32_t* out4 = nullptr;
+    int V = 0;
+};
+
 static int replay_common(hipStream_t st, int n_layers, const void* const* tape, int tape_dtype,
                          const void* const* k, const void* const* g, int in_dtype, int g_ndim,
                          const void* const* state_in, void* const* state_out, int state_dtype,
                          const void* mask, int mask_dtype, int steps, const int32_t* steps_dev, int skip_if_full,
-                         int B, int T_tape, int Hk, int Hv, int Dk, int Dv) {
+                         int B, int T_tape, int Hk, int Hv, int Dk, int Dv, const FusedAccept& acc = FusedAccept()) {
     int rc = ensure_init();
     if (rc) return rc;
     DFLASH_REQUIRE(n_layers >= 1 && n_layers <= DFLASH_MAX_BATCHED_LAYERS, "tape replay: n_layers=%d out of range", n_layers);
@@ -224,6 +262,7 @@ static int replay_common(hipStream_t st, int n_layers, const void* const* tape, 
     }
     ReplayArgs A;
     A.mask = mask; A.steps_dev = steps_dev; A.mask_dtype = mask_dtype; A.tape_dtype = tape_dtype;
+    A.verify_ids = acc.verify_ids; A.posterior = acc.posterior; A.start_inout = acc.start_inout; A.out4 = acc.out4; A.V = acc.V;
     A.in_dtype = in_dtype; A.steps = steps; A.skip_if_full = skip_if_full;
     A.T_tape = T_tape; A.Hk = Hk; A.Hv = Hv; A.Dv = Dv;
 
@@ -752,6 +791,22 @@ extern "C" int dflash_tape_replay_batched(void* stream, int n_layers, const void
     DFLASH_REQUIRE(tape && k && g && state_in && state_out, "tape replay (batched): null pointer array");
     return replay_common((hipStream_t)stream, n_layers, tape, tape_dtype, k, g, in_dtype, g_ndim, state_in, state_out,
                          state_dtype, nullptr, 0, steps, steps_dev, skip_if_full, B, T_tape, Hk, Hv, Dk, Dv);
+}
+
+extern "C" int dflash_accept_commit_replay_batched(void* stream, const uint32_t* verify_ids, const uint32_t* posterior,
+                                                   int V, int32_t* start_inout, int32_t* out4, int n_layers,
+                                                   const void* const* tape, int tape_dtype, const void* const* k,
+                                                   const void* const* g, int in_dtype, int g_ndim,
+                                                   const void* const* state_in, void* const* state_out,
+                                                   int state_dtype, int skip_if_full, int B, int T_tape, int Hk, int Hv,
+                                                   int Dk, int Dv) {
+    DFLASH_REQUIRE(verify_ids && posterior && out4 && V >= 1, "accept + replay: bad acceptance arguments");
+    DFLASH_REQUIRE(V - 1 <= T_tape, "accept + replay: %d verify positions for a tape of %d steps", V, T_tape);
+    DFLASH_REQUIRE(tape && k && g && state_in && state_out, "accept + replay: null pointer array");
+    FusedAccept acc;
+    acc.verify_ids = verify_ids; acc.posterior = posterior; acc.start_inout = start_inout; acc.out4 = out4; acc.V = V;
+    return replay_common((hipStream_t)stream, n_layers, tape, tape_dtype, k, g, in_dtype, g_ndim, state_in, state_out,
+                         state_dtype, nullptr, 0, 0, nullptr, skip_if_full, B, T_tape, Hk, Hv, Dk, Dv, acc);
 }
 
 extern "C" int dflash_gated_delta_tape(void* stream, const void* q, const void* k, const void* v, const void* g,

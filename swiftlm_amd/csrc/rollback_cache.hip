@@ -67,9 +67,17 @@ int prepare_rollback(dflash_cache* c, int n_accepted, ReplayJob* job, bool* need
                    "rollback: slot 1 still holds the pre-verify buffer; the forward must write a new one");
     int steps = n_accepted + 1;                                   // :115
     if (steps > c->T) steps = c->T;                               // slices clamp to the recorded length
-    if (c->qkv && c->keep > 0)
-        DFLASH_REQUIRE(post0 && post0 != c->snap[0] && post0 != c->qkv,
-                       "rollback: slot 0 must be a conv buffer distinct from the snapshot and from qkv");
+    if (c->qkv && c->keep > 0) {
+        // The rebuilt window is written into the post-verify conv buffer while snapshot and qkv are read:
+        // the three must not share memory (a slice of qkv handed over as the window is a view of it).
+        const size_t win = (size_t)c->B * c->keep * c->C * c->qkv_elem_bytes;
+        const size_t tape_bytes = (size_t)c->B * c->T * c->C * c->qkv_elem_bytes;
+        const uintptr_t o = (uintptr_t)post0, q = (uintptr_t)c->qkv, sn = (uintptr_t)c->snap[0];
+        const bool hits_qkv = o < q + tape_bytes && q < o + win;
+        const bool hits_snap = sn && o < sn + win && sn < o + win;
+        DFLASH_REQUIRE(post0 && !hits_qkv && !hits_snap,
+                       "rollback: slot 0 must be a conv buffer that shares no memory with the snapshot or with qkv");
+    }
     job->c = c; job->post_state = post1; job->post_conv = post0; job->steps = steps;
     *need_replay = true;
     return DFLASH_OK;

@@ -65,6 +65,7 @@ class HybridVerifyStack:
     def __init__(self, cfg: StackConfig, seed: int = 0, device: str = "cuda"):
         self.cfg = cfg
         self.lib = _lib.load()
+        self.fuse_accept = True      # acceptance decided inside the batched replay launch (one launch fewer per step)
         g = torch.Generator(device=device).manual_seed(seed)
         bf = torch.bfloat16
         T = cfg.block
@@ -147,6 +148,19 @@ class HybridVerifyStack:
                     _p(l["lse"]), _lib.BF16, self.scale, 1, cfg.Hq, cfg.Hkv, T, self.n_max, cfg.D, cfg.Hkv * hs, hs,
                     _p(self.offset), _p(self.workspace), self.workspace.numel())
                 _lib.check(rc, "sdpa_block_causal")
+        cast = lambda a: C.cast(a, _lib.vpp)
+        if self.gdn and self.fuse_accept:
+            # acceptance + rollback of every GatedDelta layer in ONE launch: the replay kernel counts the
+            # leading matches itself, writes accept[0..3] and advances the offset
+            tb = self._tables[ph]
+            note("tape_replay")
+            rc = lib.dflash_accept_commit_replay_batched(
+                st, _p(self.verify_ids[ph]), _p(self.posterior[ph]), T, _p(self.offset), _p(self.accept),
+                len(self.gdn), cast(tb["tape"]), _lib.F32, cast(tb["k"]), cast(tb["g"]), _lib.BF16, 3,
+                cast(tb["sin"]), cast(tb["sout"]), _lib.F32, 1, 1, T, cfg.Hk, cfg.Hv, cfg.Dk, cfg.Dv)
+            _lib.check(rc, "accept_commit_replay_batched")
+            self.phase = 1 - ph
+            return
         # accept: commit count -> accept[1]; offset += commit count
         rc = lib.dflash_accept_commit(st, _p(self.verify_ids[ph]), _p(self.posterior[ph]), T, _p(self.offset),
                                       _p(self.accept))
@@ -154,7 +168,6 @@ class HybridVerifyStack:
         # rollback: every GatedDelta layer in one launch, step count read on the device
         if self.gdn:
             tb = self._tables[ph]
-            cast = lambda a: C.cast(a, _lib.vpp)
             note("tape_replay")
             rc = lib.dflash_tape_replay_batched(
                 st, len(self.gdn), cast(tb["tape"]), _lib.F32, cast(tb["k"]), cast(tb["g"]), _lib.BF16, 3,

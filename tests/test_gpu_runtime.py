@@ -126,7 +126,8 @@ def _forward_into_cache(cache, d, qkv, K):
     q, k, v, g, beta = (dev(d[n], torch.bfloat16) for n in ("q", "k", "v", "g", "beta"))
     y, s_new, tape = K.gated_delta_kernel_with_tape(q, k, v, g, beta, cache[1])
     cache[1] = s_new                                           # post-verify state: a new buffer
-    cache[0] = qkv[:, -3:].contiguous()                        # post-verify conv window
+    cache[0] = qkv[:, -3:].clone()                             # post-verify conv window: its own buffer (for B = 1
+                                                               # .contiguous() would hand back a view of qkv)
     cache.record_tape(tape, k, g, qkv)
     return tape
 
@@ -160,6 +161,27 @@ def test_recurrent_rollback_cache_cycle(gpu_lib, n_accepted):
     oc.rollback(n_accepted, dtype=np.float64)
     np.testing.assert_allclose(host(cache[1]), oc.slots[1], **STATE_TOL)
     assert np.array_equal(host(cache[0]), oc.slots[0])         # conv window: bit-exact copy
+
+
+def test_rollback_refuses_a_conv_window_that_is_a_view_of_qkv(gpu_lib):
+    """The rebuilt window is written in place while qkv is read: a window that shares memory with qkv
+    is rejected instead of racing."""
+    from swiftlm_amd import DFlashKernels as K, DFlashError, RecurrentRollbackCache
+
+    B, T, Hk, Hv, Dk, Dv, Cc = 1, 16, 2, 4, 64, 32, 512
+    d = O.make_gdn_inputs(51, B, T, Hk, Hv, Dk, Dv, in_dtype="bf16")
+    cache = RecurrentRollbackCache()
+    cache[0] = torch.zeros(B, 3, Cc, dtype=torch.bfloat16, device="cuda")
+    cache[1] = dev(d["state"])
+    cache.arm_rollback(prefix_len=0)
+    qkv = torch.randn(B, T, Cc, device="cuda").bfloat16()
+    q, k, v, g, beta = (dev(d[n], torch.bfloat16) for n in ("q", "k", "v", "g", "beta"))
+    y, s_new, tape = K.gated_delta_kernel_with_tape(q, k, v, g, beta, cache[1])
+    cache[1] = s_new
+    cache[0] = qkv[:, -3:]                                     # a view of the tape's qkv
+    cache.record_tape(tape, k, g, qkv)
+    with pytest.raises(DFlashError):
+        cache.rollback(3)
 
 
 def test_restore_target_cache_hybrid_stack(gpu_lib):
@@ -284,3 +306,46 @@ def test_plain_c_client_of_the_abi(gpu_lib):
     r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
     assert r.returncode == 0, r.stdout + r.stderr
     assert "C ABI check passed" in r.stdout
+
+
+# ---- the verify-step driver (what bench.py times): fused and unfused acceptance agree, both match the oracle ----
+
+def test_verify_stack_steps_match_oracle_and_fused_accept(gpu_lib):
+    import torch
+    from swiftlm_amd.verify_step import HybridVerifyStack, StackConfig
+
+    cfg = StackConfig(n_layers=8, attn_every=4, block=16, Hk=2, Hv=4, Dk=128, Dv=32, Hq=4, Hkv=2, D=128,
+                      context=150, max_steps=6)
+    stacks = [HybridVerifyStack(cfg, seed=3), HybridVerifyStack(cfg, seed=3)]
+    stacks[0].fuse_accept, stacks[1].fuse_accept = True, False
+    commits = [3, 16, 1, 9]
+    offset = cfg.context
+    for step, cc in enumerate(commits):
+        pre = None
+        for st in stacks:
+            ph = st.phase
+            st.set_acceptance(ph, cc, seed=step)
+            if pre is None:
+                pre = [dict(state=host(l["state"][ph])) for l in st.gdn]
+            st.enqueue_step()
+        torch.cuda.synchronize()
+        offset += cc
+        a, b = stacks
+        assert a.accept.tolist() == b.accept.tolist() == [cc - 1, cc, int(a.posterior[1 - a.phase][cc - 1]), offset]
+        assert int(a.offset) == int(b.offset) == offset
+        for la, lb, p0 in zip(a.gdn, b.gdn, pre):
+            post = 1 - (1 - a.phase)          # the buffer the step wrote = the new pre-verify state = state[a.phase]
+            assert torch.equal(la["state"][a.phase], lb["state"][b.phase])
+            assert torch.equal(la["tape"], lb["tape"]) and torch.equal(la["y"], lb["y"])
+            # oracle: forward on the block, then (unless everything was accepted) replay of cc steps
+            yw, sw, tw = O.gated_delta_ops_with_tape(host(la["q"]), host(la["k"]), host(la["v"]), host(la["g"]),
+                                                      host(la["beta"]), p0["state"])
+            want = sw if cc == cfg.block else O.tape_replay_ops(tw[:, :cc].astype(np.float32), host(la["k"])[:, :cc],
+                                                                host(la["g"])[:, :cc], p0["state"])
+            np.testing.assert_allclose(host(la["state"][a.phase]), want, **STATE_TOL)
+        for la, lb in zip(a.attn, b.attn):
+            assert torch.equal(la["out"], lb["out"])
+            n_keys = offset - cc + cfg.block
+            ow, _ = O.sdpa_block_causal(host(la["q"]), host(la["k_cache"])[:, :, :n_keys], host(la["v_cache"])[:, :, :n_keys],
+                                        a.scale)
+            np.testing.assert_allclose(host(la["out"]), ow, rtol=2e-2, atol=2e-2)
