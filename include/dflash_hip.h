@@ -222,6 +222,37 @@ int dflash_sdpa_block_causal_append(void* stream,
                                     const int32_t* cache_len_dev,
                                     void* workspace, size_t workspace_bytes);
 
+/* The same attention over a PAGED K/V cache.  The reference's cache is one dense
+ * [B, Hk, N, D] array per layer (KVCacheSimple in mlx-swift-lm; the attention reads it
+ * as DFlashKernels.swift:737-743 receives it), so paging has no counterpart there: the
+ * entry computes exactly what dflash_sdpa_block_causal / _append compute on the dense
+ * array that gathering the pages would give, bit for bit.
+ *
+ * k_pool, v_pool hold num_pages pages; page p, head h, row r, channel d sits at element
+ * p * page_stride + h * head_stride + r * D + d (head_stride >= page_size * D, page_stride
+ * >= (Hk-1) * head_stride + page_size * D, both multiples of 8).  page_size is a power of
+ * two >= 32.  Key n of sequence b lives in page page_table[b * page_table_stride + n /
+ * page_size] (device int32; page_table_stride * page_size >= N), row n % page_size.  Entries
+ * are clamped to [0, num_pages) on the device, so a stale table cannot address outside the pool.
+ *
+ * k_new == v_new == NULL: plain attention, len_dev as kv_len_dev above (keys per sequence,
+ * block included).  Otherwise k_new, v_new [B, Hk, M, D] are the block's rows as in the
+ * append entry: read from there, stored into the pages that hold keys len..len+M-1 (which
+ * the table must already map), and len_dev counts the rows already cached, block excluded.
+ * No additive mask.  Returns DFLASH_NOT_SUPPORTED for a page size the kernel does not
+ * take or a sequence so long that one workgroup's span exceeds 512 pages.
+ * ---------------------------------------------------------------------- */
+int dflash_sdpa_block_causal_paged(void* stream,
+                                   const void* q, void* k_pool, void* v_pool,
+                                   const int32_t* page_table, int page_table_stride,
+                                   int page_size, int num_pages,
+                                   int64_t page_stride, int64_t head_stride,
+                                   const void* k_new, const void* v_new,
+                                   void* out, float* lse, int dtype, float scale,
+                                   int B, int Hq, int Hk, int M, int N, int D,
+                                   const int32_t* len_dev,
+                                   void* workspace, size_t workspace_bytes);
+
 /* ------------------------------------------------------------------------
  * Acceptance.  dflash_match_acceptance_length replaces
  * DFlashRuntime.matchAcceptanceLength (Sources/DFlash/DFlashRuntime.swift:

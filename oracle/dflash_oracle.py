@@ -472,6 +472,30 @@ def sdpa_block_causal(q, k, v, scale, mask=None, *, dtype=np.float64):
     return out, lse
 
 
+def gather_pages(pool, page_table, n_keys: int):
+    """Dense [B, Hk, n_keys, D] view of a paged cache: pool [num_pages, Hk, page_size, D],
+    page_table [B, pages]; key n of sequence b is row n % page_size of page page_table[b, n // page_size].
+    The reference keeps its cache dense (what batchedSDPA2Pass receives, DFlashKernels.swift:737-743);
+    this is the layout transform that relates the paged entry to it."""
+    pool = np.asarray(pool)
+    page_table = np.asarray(page_table)
+    ps = pool.shape[2]
+    n = np.arange(n_keys)
+    pages = page_table[:, n // ps]                      # [B, n_keys]
+    return np.transpose(pool[pages, :, (n % ps)[None, :]], (0, 2, 1, 3))
+
+
+def scatter_pages(dense, page_table, num_pages: int, page_size: int, fill=0.0):
+    """Inverse of gather_pages: a pool that holds dense [B, Hk, N, D] under page_table."""
+    dense = np.asarray(dense)
+    B, Hk, N, D = dense.shape
+    pool = np.full((num_pages, Hk, page_size, D), fill, dtype=dense.dtype)
+    for b in range(B):
+        for n in range(N):
+            pool[page_table[b][n // page_size], :, n % page_size] = dense[b, :, n]
+    return pool
+
+
 def sdpa_2pass(q, k, v, scale, blocks=32, *, partial_dtype="bf16"):
     """Restatement of the reference's split-KV two-pass kernels in float32.
 

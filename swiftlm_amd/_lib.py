@@ -37,6 +37,8 @@ SIGNATURES = {
     "dflash_sdpa_block_causal": (i32, [vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp, vp, sz]),
     "dflash_sdpa_block_causal_masked": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp, vp, sz]),
     "dflash_sdpa_block_causal_append": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp, vp, sz]),
+    "dflash_sdpa_block_causal_paged": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, i64, i64, vp, vp, vp, vp, i32, f32] + [i32] * 6 +
+                                       [vp, vp, sz]),
     "dflash_match_acceptance_length": (i32, [vp, vp, vp, i32, vp]),
     "dflash_accept_commit": (i32, [vp, vp, vp, i32, vp, vp]),
     "dflash_accept_commit_replay_batched": (i32, [vp, vp, vp, i32, vp, vp, i32, vpp, i32, vpp, vpp, i32, i32, vpp, vpp, i32,

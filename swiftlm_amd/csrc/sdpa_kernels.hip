@@ -94,7 +94,14 @@ struct SdpaArgs {
     int Hq, Hk, G, N, S, groups_per_kv;
     int rows_total;     // B*Hq*16
     int len_bias;       // added to kv_len_dev[b]: 0, or 16 when the device count excludes the block
+    // Paged K/V (PAGED instantiations): key n of sequence b lives in page page_table[b * table_stride + (n >> page_shift)]
+    // of the pool, at row n & (page_size - 1); k, v point at the pools, kv_batch_stride is the page pitch and
+    // kv_head_stride the head pitch inside a page.
+    const int32_t* page_table;
+    int page_shift, table_stride, num_pages;
 };
+
+constexpr int kPageSlots = 512;     // page-table entries one workgroup keeps in LDS (its own span of the sequence)
 
 // LDS plan of the partial kernel.  A stage holds one tile of kBN keys: the K rows
 // followed by the V rows, both row-major [key][D] exactly as in HBM but with the
@@ -167,7 +174,7 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 // and its mask value is at least the lowest finite value of the input type, and the mask value is
 // added to the scaled score (DFlashKernels.swift:550-553, :614-623).  The mask is read with plain
 // loads inside the softmax; that instantiation is for signature parity, not for speed.
-template <typename Tag, int D, bool MASKED>
+template <typename Tag, int D, bool MASKED, bool PAGED>
 __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs A) {
     typedef typename Tag::vec8 vec8;
     typedef SdpaLds<D> L;
@@ -202,10 +209,23 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
     const int qi = c & 15;
     const size_t row_id = ((size_t)b * A.Hq + hq) * kM + qi;   // valid only when row_valid
 
-    const unsigned char* kbase = reinterpret_cast<const unsigned char*>(A.k) +
-                                 ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
-    const unsigned char* vbase = reinterpret_cast<const unsigned char*>(A.v) +
-                                 ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
+    // dense: the head's rows are contiguous; paged: the head's slice of page 0, pages are added per tile
+    const size_t head_off = PAGED ? (size_t)hk * A.kv_head_stride * 2
+                                  : ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
+    const unsigned char* kbase = reinterpret_cast<const unsigned char*>(A.k) + head_off;
+    const unsigned char* vbase = reinterpret_cast<const unsigned char*>(A.v) + head_off;
+    // Paged: byte offset of key n's row from kbase / vbase.  The entries of this workgroup's span are kept
+    // in LDS behind the tile ring (filled below, once the span is known); entries are clamped to the pool.
+    int32_t* ptab = reinterpret_cast<int32_t*>(smem + L::BYTES);
+    const int page_mask = PAGED ? (1 << A.page_shift) - 1 : 0;
+    int page0 = 0;                                      // first page of this workgroup's span
+    auto clamp_page = [&](int e) { return e < 0 ? 0 : (e >= A.num_pages ? A.num_pages - 1 : e); };
+    auto row_off = [&](int key) -> size_t {
+        if constexpr (PAGED)
+            return (size_t)ptab[(key >> A.page_shift) - page0] * (size_t)A.kv_batch_stride * 2 + (size_t)(key & page_mask) * L::ROWB;
+        else
+            return (size_t)key * L::ROWB;
+    };
 
     // Fused append: keys Nb-16 .. Nb-1 are read from k_new / v_new, and one workgroup per KV head
     // stores them into the cache rows they stand for.
@@ -214,12 +234,25 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
     const unsigned char* knew = reinterpret_cast<const unsigned char*>(A.k_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
     const unsigned char* vnew = reinterpret_cast<const unsigned char*>(A.v_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
     if (fused && A.k_cache && split == 0 && hg0 == 0) {
-        const size_t head = ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2 + (size_t)cache_rows * L::ROWB;
-        u32x4_t* kd = reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.k_cache) + head);
-        u32x4_t* vd = reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.v_cache) + head);
         const u32x4_t* ksrc = reinterpret_cast<const u32x4_t*>(knew);
         const u32x4_t* vsrc = reinterpret_cast<const u32x4_t*>(vnew);
-        for (int i = tid; i < kM * L::CPR; i += kSdpaThreads) { kd[i] = ksrc[i]; vd[i] = vsrc[i]; }
+        if constexpr (PAGED) {
+            // the 16 rows may straddle a page boundary: each row looks its page up (read from the table itself:
+            // this workgroup's LDS span covers the start of the sequence, not its end)
+            for (int i = tid; i < kM * L::CPR; i += kSdpaThreads) {
+                const int key = cache_rows + i / L::CPR;
+                const int page = clamp_page(A.page_table[(size_t)b * A.table_stride + (key >> A.page_shift)]);
+                const size_t off = head_off + (size_t)page * (size_t)A.kv_batch_stride * 2 + (size_t)(key & page_mask) * L::ROWB +
+                                   (size_t)(i % L::CPR) * 16;
+                *reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.k_cache) + off) = ksrc[i];
+                *reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.v_cache) + off) = vsrc[i];
+            }
+        } else {
+            const size_t head = head_off + (size_t)cache_rows * L::ROWB;
+            u32x4_t* kd = reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.k_cache) + head);
+            u32x4_t* vd = reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.v_cache) + head);
+            for (int i = tid; i < kM * L::CPR; i += kSdpaThreads) { kd[i] = ksrc[i]; vd[i] = vsrc[i]; }
+        }
     }
 
     if (t_begin >= t_end) {   // empty split: tell the combine kernel to ignore it
@@ -228,6 +261,16 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
             A.part_l[row_id * A.S + split] = 0.f;
         }
         return;
+    }
+
+    if constexpr (PAGED) {
+        // this workgroup's keys t_begin*kBN .. min(t_end*kBN, Nb) - 1 and the pages they live in
+        page0 = (t_begin * kBN) >> A.page_shift;
+        const int last_key = (t_end * kBN < Nb ? t_end * kBN : Nb) - 1;
+        int npg = (last_key >> A.page_shift) - page0 + 1;                // the host checks that the span fits
+        npg = npg < kPageSlots ? npg : kPageSlots;
+        for (int i = tid; i < npg; i += kSdpaThreads) ptab[i] = clamp_page(A.page_table[(size_t)b * A.table_stride + page0 + i]);
+        __syncthreads();
     }
 
     // ---- asynchronous tile loads ------------------------------------------------
@@ -249,8 +292,9 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
         const int key0 = t * kBN;
         const int rg = (4 * j + wave) * L::RPI;
         if (key0 + kBN <= cache_rows) {          // uniform: whole tile comes from the cache
-            const unsigned char* kt = uniform_ptr(kbase + (size_t)key0 * L::ROWB);
-            const unsigned char* vt = uniform_ptr(vbase + (size_t)key0 * L::ROWB);
+            const size_t toff = row_off(key0);   // a tile never straddles a page (page sizes are multiples of kBN)
+            const unsigned char* kt = uniform_ptr(kbase + toff);
+            const unsigned char* vt = uniform_ptr(vbase + toff);
             async_load_16B(kt, ld_off_k[j], stage_lds + rg * L::ROWB);
             async_load_16B(vt, ld_off_v[j], stage_lds + L::K_BYTES + rg * L::ROWB);
         } else {
@@ -261,10 +305,9 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
             key = key < Nb ? key : Nb - 1;
             const uint32_t pk = (uint32_t)((ld_pos ^ (row & 15)) * 16);
             const uint32_t pv = (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
-            const unsigned char* ksrc = key < cache_rows ? kbase + (size_t)key * L::ROWB
-                                                          : knew + (size_t)(key - cache_rows) * L::ROWB;
-            const unsigned char* vsrc = key < cache_rows ? vbase + (size_t)key * L::ROWB
-                                                          : vnew + (size_t)(key - cache_rows) * L::ROWB;
+            const size_t roff = row_off(key < cache_rows ? key : (cache_rows > 0 ? cache_rows - 1 : 0));
+            const unsigned char* ksrc = key < cache_rows ? kbase + roff : knew + (size_t)(key - cache_rows) * L::ROWB;
+            const unsigned char* vsrc = key < cache_rows ? vbase + roff : vnew + (size_t)(key - cache_rows) * L::ROWB;
             async_load_16B_addr(ksrc + pk, stage_lds + rg * L::ROWB);
             async_load_16B_addr(vsrc + pv, stage_lds + L::K_BYTES + rg * L::ROWB);
         }
@@ -385,8 +428,9 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
         constexpr bool kIssue = decltype(with_issue)::value;
         // the requested tile lies entirely inside the cache: only scalar bases move
         const uint32_t is_lds = smem_lds + ((t_issue - t_begin) % kStages) * L::STAGE;
-        const unsigned char* is_k = uniform_ptr(kbase + (size_t)t_issue * kBN * L::ROWB);
-        const unsigned char* is_v = uniform_ptr(vbase + (size_t)t_issue * kBN * L::ROWB);
+        const size_t is_off = kIssue ? row_off(t_issue * kBN) : 0;
+        const unsigned char* is_k = uniform_ptr(kbase + is_off);
+        const unsigned char* is_v = uniform_ptr(vbase + is_off);
         const unsigned char* ks = stage_of(t + 1);
         const float m_safe = m_run == -INFINITY ? 0.f : m_run;
         float psum = 0.f;
@@ -745,19 +789,20 @@ static size_t ws_layout(int B, int Hq, int S, int D, size_t* off_m, size_t* off_
     return (o + 255) & ~(size_t)255;
 }
 
-template <typename Tag, int D, bool MASKED>
+template <typename Tag, int D, bool MASKED, bool PAGED>
 static int launch_sdpa(hipStream_t st, const SdpaArgs& A, const CombineArgs& C, int B) {
     typedef SdpaLds<D> L;
-    static_assert(L::BYTES <= 160 * 1024, "tile buffers must fit the 160 KB LDS of a gfx950 CU");
-    auto kern = sdpa_partial_kernel<Tag, D, MASKED>;
+    constexpr int kLdsBytes = L::BYTES + (PAGED ? kPageSlots * (int)sizeof(int32_t) : 0);
+    static_assert(kLdsBytes <= 160 * 1024, "tile buffers must fit the 160 KB LDS of a gfx950 CU");
+    auto kern = sdpa_partial_kernel<Tag, D, MASKED, PAGED>;
     // Raise the dynamic LDS limit above the 64 KB default, once per process.
     static const hipError_t attr_rc =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::BYTES);
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     DFLASH_HIP_TRY(attr_rc);
     dim3 grid(A.S, A.Hk * A.groups_per_kv, B);
     {
         LaunchBracket br(DFLASH_KERNEL_SDPA_PARTIAL, st);
-        br.launch(kern, grid, dim3(kSdpaThreads), L::BYTES, A);
+        br.launch(kern, grid, dim3(kSdpaThreads), kLdsBytes, A);
     }
     DFLASH_HIP_TRY(hipGetLastError());
     {
@@ -781,10 +826,16 @@ extern "C" size_t dflash_sdpa_workspace_bytes(int B, int Hq, int Hk, int M, int 
     return ws_layout(B, Hq, choose_splits(B, Hk, groups, N), D, &om, &ol);
 }
 
+// Page table of a paged K/V pool (null for the dense layout): kv_batch_stride is then the page pitch.
+struct PagedKv {
+    const int32_t* table;
+    int table_stride, page_size, num_pages;
+};
+
 static int sdpa_common(void* stream, const void* q, const void* k, const void* v, const void* k_new, const void* v_new,
                        void* k_cache, void* v_cache, const void* mask, void* out, float* lse, int dtype, float scale, int B, int Hq, int Hk,
                        int M, int N, int D, int64_t kv_batch_stride, int64_t kv_head_stride, const int32_t* kv_len_dev,
-                       void* workspace, size_t workspace_bytes) {
+                       void* workspace, size_t workspace_bytes, const PagedKv* paged = nullptr) {
     int rc = ensure_init();
     if (rc) return rc;
     DFLASH_REQUIRE(q && k && v && out, "sdpa: null pointer");
@@ -795,9 +846,23 @@ static int sdpa_common(void* stream, const void* q, const void* k, const void* v
     DFLASH_SUPPORTED(D == 128 || D == 256, "sdpa: head dim %d is not 128 or 256", D);
     DFLASH_SUPPORTED(Hq % Hk == 0, "sdpa: Hq=%d is not a multiple of Hk=%d", Hq, Hk);
     DFLASH_REQUIRE(N >= M, "sdpa: N=%d must include the %d block tokens", N, M);
-    DFLASH_REQUIRE(kv_head_stride >= (int64_t)N * D, "sdpa: kv_head_stride smaller than N*D");
-    DFLASH_REQUIRE((int64_t)N * D * 2 < (1LL << 32), "sdpa: one KV head of %d keys exceeds the 4 GiB the kernel addresses", N);
-    DFLASH_REQUIRE(kv_batch_stride >= (int64_t)(Hk - 1) * kv_head_stride + (int64_t)N * D, "sdpa: kv_batch_stride too small");
+    int page_shift = 0;
+    if (paged) {
+        DFLASH_REQUIRE(paged->table != nullptr, "sdpa (paged): null page table");
+        DFLASH_SUPPORTED(!mask, "sdpa (paged): the additive mask is not supported with paged K/V");
+        const int ps = paged->page_size;
+        DFLASH_SUPPORTED(ps >= kBN && (ps & (ps - 1)) == 0, "sdpa (paged): page size %d is not a power of two >= %d", ps, kBN);
+        while ((1 << page_shift) < ps) ++page_shift;
+        DFLASH_REQUIRE(paged->num_pages > 0, "sdpa (paged): empty pool");
+        DFLASH_REQUIRE((int64_t)paged->table_stride * ps >= N, "sdpa (paged): %d table entries of %d keys do not cover N=%d",
+                       paged->table_stride, ps, N);
+        DFLASH_REQUIRE(kv_head_stride >= (int64_t)ps * D, "sdpa (paged): head pitch smaller than page_size*D");
+        DFLASH_REQUIRE(kv_batch_stride >= (int64_t)(Hk - 1) * kv_head_stride + (int64_t)ps * D, "sdpa (paged): page pitch too small");
+    } else {
+        DFLASH_REQUIRE(kv_head_stride >= (int64_t)N * D, "sdpa: kv_head_stride smaller than N*D");
+        DFLASH_REQUIRE((int64_t)N * D * 2 < (1LL << 32), "sdpa: one KV head of %d keys exceeds the 4 GiB the kernel addresses", N);
+        DFLASH_REQUIRE(kv_batch_stride >= (int64_t)(Hk - 1) * kv_head_stride + (int64_t)N * D, "sdpa: kv_batch_stride too small");
+    }
     DFLASH_REQUIRE(kv_head_stride % 8 == 0 && kv_batch_stride % 8 == 0, "sdpa: kv strides must be multiples of 8 elements");
     DFLASH_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out | (uintptr_t)k_new | (uintptr_t)v_new) % 16 == 0,
                    "sdpa: q/k/v/out must be 16-byte aligned");
@@ -806,6 +871,12 @@ static int sdpa_common(void* stream, const void* q, const void* k, const void* v
     const int G = Hq / Hk;
     const int groups = (G + kHeadsPerWG - 1) / kHeadsPerWG;
     const int S = choose_splits(B, Hk, groups, N);
+    if (paged) {
+        const int nt = (N + kBN - 1) / kBN;
+        const int span_pages = ((((nt + S - 1) / S) * kBN) >> page_shift) + 2;      // pages one workgroup's keys can touch
+        DFLASH_SUPPORTED(span_pages <= kPageSlots, "sdpa (paged): %d pages per workgroup exceed the %d the kernel keeps", span_pages,
+                         kPageSlots);
+    }
     size_t om, ol;
     const size_t need = ws_layout(B, Hq, S, D, &om, &ol);
     DFLASH_REQUIRE(workspace && workspace_bytes >= need, "sdpa: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
@@ -824,17 +895,25 @@ static int sdpa_common(void* stream, const void* q, const void* k, const void* v
     A.scale_log2 = scale * 1.4426950408889634f;
     A.Hq = Hq; A.Hk = Hk; A.G = G; A.N = N; A.S = S; A.groups_per_kv = groups; A.rows_total = B * Hq * kM;
     A.len_bias = k_new ? kM : 0;
+    A.page_table = paged ? paged->table : nullptr;
+    A.page_shift = page_shift;
+    A.table_stride = paged ? paged->table_stride : 0;
+    A.num_pages = paged ? paged->num_pages : 0;
     CombineArgs C;
     C.part_o = A.part_o; C.part_m = A.part_m; C.part_l = A.part_l;
     C.out = (uint16_t*)out; C.lse = lse; C.S = S;
 
     hipStream_t st = (hipStream_t)stream;
     if (mask) {
-        if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa<Bf16Tag, 256, true>(st, A, C, B) : launch_sdpa<Bf16Tag, 128, true>(st, A, C, B);
-        return D == 256 ? launch_sdpa<F16Tag, 256, true>(st, A, C, B) : launch_sdpa<F16Tag, 128, true>(st, A, C, B);
+        if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa<Bf16Tag, 256, true, false>(st, A, C, B) : launch_sdpa<Bf16Tag, 128, true, false>(st, A, C, B);
+        return D == 256 ? launch_sdpa<F16Tag, 256, true, false>(st, A, C, B) : launch_sdpa<F16Tag, 128, true, false>(st, A, C, B);
     }
-    if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa<Bf16Tag, 256, false>(st, A, C, B) : launch_sdpa<Bf16Tag, 128, false>(st, A, C, B);
-    return D == 256 ? launch_sdpa<F16Tag, 256, false>(st, A, C, B) : launch_sdpa<F16Tag, 128, false>(st, A, C, B);
+    if (paged) {
+        if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa<Bf16Tag, 256, false, true>(st, A, C, B) : launch_sdpa<Bf16Tag, 128, false, true>(st, A, C, B);
+        return D == 256 ? launch_sdpa<F16Tag, 256, false, true>(st, A, C, B) : launch_sdpa<F16Tag, 128, false, true>(st, A, C, B);
+    }
+    if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa<Bf16Tag, 256, false, false>(st, A, C, B) : launch_sdpa<Bf16Tag, 128, false, false>(st, A, C, B);
+    return D == 256 ? launch_sdpa<F16Tag, 256, false, false>(st, A, C, B) : launch_sdpa<F16Tag, 128, false, false>(st, A, C, B);
 }
 
 extern "C" int dflash_sdpa_block_causal(void* stream, const void* q, const void* k, const void* v, void* out,
@@ -863,4 +942,16 @@ extern "C" int dflash_sdpa_block_causal_masked(void* stream, const void* q, cons
     DFLASH_REQUIRE(mask, "sdpa (masked): null mask");
     return sdpa_common(stream, q, k, v, nullptr, nullptr, nullptr, nullptr, mask, out, lse, dtype, scale, B, Hq, Hk, M, N, D,
                        kv_batch_stride, kv_head_stride, kv_len_dev, workspace, workspace_bytes);
+}
+
+extern "C" int dflash_sdpa_block_causal_paged(void* stream, const void* q, void* k_pool, void* v_pool,
+                                              const int32_t* page_table, int page_table_stride, int page_size, int num_pages,
+                                              int64_t page_stride, int64_t head_stride, const void* k_new, const void* v_new,
+                                              void* out, float* lse, int dtype, float scale, int B, int Hq, int Hk, int M, int N,
+                                              int D, const int32_t* len_dev, void* workspace, size_t workspace_bytes) {
+    DFLASH_REQUIRE(k_pool && v_pool, "sdpa (paged): null pool");
+    DFLASH_REQUIRE((k_new == nullptr) == (v_new == nullptr), "sdpa (paged): k_new and v_new go together");
+    PagedKv pg{page_table, page_table_stride, page_size, num_pages};
+    return sdpa_common(stream, q, k_pool, v_pool, k_new, v_new, k_new ? k_pool : nullptr, k_new ? v_pool : nullptr, nullptr, out, lse,
+                       dtype, scale, B, Hq, Hk, M, N, D, page_stride, head_stride, len_dev, workspace, workspace_bytes, &pg);
 }

@@ -287,6 +287,63 @@ class DFlashKernels:
         return (out, lse) if return_lse else out
 
     @staticmethod
+    def batched_sdpa_2pass_paged(queries: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                                 page_table: torch.Tensor, scale: float, n_keys: int, *,
+                                 k_new: Optional[torch.Tensor] = None, v_new: Optional[torch.Tensor] = None,
+                                 lengths: Optional[torch.Tensor] = None, return_lse: bool = False,
+                                 workspace: Optional[torch.Tensor] = None):
+        """The verify block's attention over a paged K/V cache.  ``k_pool``/``v_pool``
+        [num_pages, Hk, page_size, D] (page_size a power of two >= 32); ``page_table`` int32
+        [B, pages_per_sequence] maps key n of sequence b to page ``page_table[b, n // page_size]``.
+        Without ``k_new``/``v_new`` this is ``batched_sdpa_2pass`` on the gathered cache (``lengths``:
+        keys per sequence, block included); with them it is ``batched_sdpa_2pass_append`` (``lengths``:
+        rows already cached, block excluded; the block's rows are stored into their pages).  The
+        reference's cache is dense (``batchedSDPA2Pass``, DFlashKernels.swift:737-743, takes one
+        [B,Hk,N,D] array), so paging has no counterpart there.  Returns None for unsupported shapes."""
+        _dev(queries, k_pool, v_pool, page_table, k_new, v_new, lengths, workspace)
+        if queries.dim() != 4 or k_pool.dim() != 4 or k_pool.shape != v_pool.shape or page_table.dim() != 2:
+            return None
+        B, Hq, M, D = queries.shape
+        num_pages, Hk, page_size = k_pool.shape[0], k_pool.shape[1], k_pool.shape[2]
+        if k_pool.shape[3] != D or k_pool.dtype != queries.dtype or v_pool.dtype != queries.dtype:
+            return None
+        if (k_new is None) != (v_new is None):
+            raise DFlashError("batched_sdpa_2pass_paged: k_new and v_new go together")
+        if k_new is not None and (k_new.shape != (B, Hk, M, D) or v_new.shape != (B, Hk, M, D)
+                                  or k_new.dtype != queries.dtype or v_new.dtype != queries.dtype):
+            return None
+        if page_table.dtype != torch.int32 or page_table.shape[0] != B or page_table.stride(1) != 1:
+            raise DFlashError("batched_sdpa_2pass_paged: page_table must be int32 [B, pages] with unit inner stride")
+        if k_pool.stride(3) != 1 or k_pool.stride(2) != D or k_pool.stride() != v_pool.stride():
+            raise DFlashError("batched_sdpa_2pass_paged: the pools must be row-contiguous and laid out alike")
+        if page_table.shape[1] * page_size < n_keys:
+            raise DFlashError(f"batched_sdpa_2pass_paged: {page_table.shape[1]} pages of {page_size} keys do not cover n_keys={n_keys}")
+        table_pitch = page_table.stride(0) if B > 1 else page_table.shape[1]      # a single row's stride means nothing
+        queries = queries.contiguous()
+        if k_new is not None:
+            k_new, v_new = k_new.contiguous(), v_new.contiguous()
+        lib = _lib.load()
+        need = int(lib.dflash_sdpa_workspace_bytes(B, Hq, Hk, M, n_keys, D))
+        if need == 0:
+            return None
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=queries.device)
+        out = torch.empty_like(queries)
+        lse = torch.empty((B, Hq, M), dtype=torch.float32, device=queries.device) if return_lse else None
+        try:
+            code = _code(queries)
+        except DFlashUnsupported:
+            return None
+        rc = lib.dflash_sdpa_block_causal_paged(
+            _stream(), _ptr(queries), _ptr(k_pool), _ptr(v_pool), _ptr(page_table), table_pitch, page_size, num_pages,
+            k_pool.stride(0), k_pool.stride(1), _ptr(k_new), _ptr(v_new), _ptr(out), _ptr(lse), code, float(scale),
+            B, Hq, Hk, M, int(n_keys), D, _ptr(lengths), _ptr(workspace), workspace.numel() * workspace.element_size())
+        if rc == _lib.UNSUPPORTED:
+            return None
+        _lib.check(rc, "batched_sdpa_2pass_paged")
+        return (out, lse) if return_lse else out
+
+    @staticmethod
     def sdpa_fallback(queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, scale: float,
                       mask: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``sdpaFallback`` (DFlashKernels.swift:818-828) delegates to the array library's
