@@ -221,3 +221,49 @@ def test_paged_rejects_what_it_does_not_take(gpu_lib):
         None, p(q), p(k_pool), p(v_pool), p(table), 4, 32, k_pool.shape[0], k_pool.stride(0), k_pool.stride(1), p(q), None,
         p(out), None, _lib.BF16, 1.0 / 16, 1, 16, 2, 16, 116, 256, None, p(ws), ws.numel())
     assert rc == _lib.INVALID
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_paged_random_shapes(gpu_lib, seed):
+    """Seeded random shapes, page sizes and ragged lengths, with and without the fused append:
+    bit-identical to the dense entries, and within tolerance of the oracle on the gathered cache."""
+    from swiftlm_amd import DFlashKernels as K
+
+    rng = np.random.default_rng(seed)
+    for it in range(20):
+        D = int(rng.choice([128, 256]))
+        Hk = int(rng.choice([1, 2, 3]))
+        Hq = Hk * int(rng.choice([1, 2, 4, 8, 9]))
+        B = int(rng.choice([1, 2, 3]))
+        P = int(rng.choice([32, 64, 128, 512]))
+        dt = torch.bfloat16 if rng.random() < 0.7 else torch.float16
+        Ls = [int(rng.choice([0, 1, 15, 16, 17, 31, 33, 100, 257, 700])) for _ in range(B)]
+        lens = [l + 16 for l in Ls]
+        append = bool(rng.random() < 0.5)
+        case = f"seed {seed} case {it}: B={B} Hq={Hq} Hk={Hk} Ls={Ls} D={D} P={P} {dt} append={append}"
+        q, k, v, k_pool, v_pool, table = paged_case(int(rng.integers(1 << 30)), B, Hq, Hk, lens, D, P, dt,
+                                                    head_pad=int(rng.choice([0, 8, 64])), page_pad=int(rng.choice([0, 16])))
+        scale = 1.0 / math.sqrt(D)
+        kv_len = torch.tensor(lens, dtype=torch.int32, device="cuda")
+        want, want_lse = K.batched_sdpa_2pass(q, k, v, scale, return_lse=True, kv_len=kv_len)
+        if append:
+            k_new = torch.stack([k[b, :, Ls[b]:Ls[b] + 16] for b in range(B)]).contiguous()
+            v_new = torch.stack([v[b, :, Ls[b]:Ls[b] + 16] for b in range(B)]).contiguous()
+            tb = table.cpu().numpy()
+            for b in range(B):
+                for n in range(Ls[b], lens[b]):
+                    k_pool[tb[b, n // P], :, n % P] = 3.0
+                    v_pool[tb[b, n // P], :, n % P] = 3.0
+            got, got_lse = K.batched_sdpa_2pass_paged(q, k_pool, v_pool, table, scale, max(lens), k_new=k_new, v_new=v_new,
+                                                      lengths=torch.tensor(Ls, dtype=torch.int32, device="cuda"), return_lse=True)
+        else:
+            got, got_lse = K.batched_sdpa_2pass_paged(q, k_pool, v_pool, table, scale, max(lens), lengths=kv_len, return_lse=True)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want) and torch.equal(got_lse, want_lse), case
+        for b in range(B):
+            kd = O.gather_pages(host(k_pool), table.cpu().numpy()[b:b + 1], lens[b])
+            vd = O.gather_pages(host(v_pool), table.cpu().numpy()[b:b + 1], lens[b])
+            assert np.array_equal(kd, host(k[b:b + 1, :, : lens[b]])) and np.array_equal(vd, host(v[b:b + 1, :, : lens[b]])), case
+            ref, ref_lse = O.sdpa_block_causal(host(q[b:b + 1]), kd, vd, scale)
+            np.testing.assert_allclose(host(got[b:b + 1]), ref, err_msg=case, **OUT_TOL)
+            np.testing.assert_allclose(host(got_lse[b:b + 1]), ref_lse, err_msg=case, **LSE_TOL)
