@@ -186,6 +186,9 @@ def main():
     ap.add_argument("--aux", action="store_true",
                     help="also time the kernels next to the measured path (pre-ops, greedy tokens) and report them "
                          "under aux_kernels; they are not part of the step time")
+    ap.add_argument("--page-size", type=int, default=0,
+                    help="keep the attention layers' K/V in paged pools with pages of this many keys (0: dense caches, "
+                         "the configuration the headline number is quoted on)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy, the known-size kernel the rocprof byte counters are scaled by")
     args = ap.parse_args()
@@ -206,7 +209,7 @@ def main():
     K, W = args.steps, args.warmup
     brk_steps = min(max(K, 1), 16)                 # eager pass with events attached to the kernels
     total = 2 + W + K + brk_steps
-    cfg = StackConfig(context=args.context, max_steps=total + 2)
+    cfg = StackConfig(context=args.context, max_steps=total + 2, page_size=args.page_size)
     stack = HybridVerifyStack(cfg, seed=0)
     T = cfg.block
     commits = draw_commit_counts(total, T)
@@ -338,6 +341,7 @@ def main():
                          "fp32 state; attention Hq=16 Hkv=2 D=256 bf16") % cfg.context,
             "layers": cfg.n_layers, "block": T, "context": cfg.context,
             "launch": "eager" if graphs is None else "hip-graph, 2 steps per graph",
+            "kv_layout": "dense" if not cfg.page_size else "paged, %d-key pages" % cfg.page_size,
         },
         "step_hbm_algorithmic_gbs": round(step_bytes / (ms_per_step * 1e-3) / 1e9, 1),
         "step_frac_of_hbm_peak": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),

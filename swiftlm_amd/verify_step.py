@@ -6,7 +6,8 @@ loop runs it (Sources/DFlash/DFlashRuntime.swift:484-581):
   1. per GatedDelta layer: forward-with-tape from the pre-verify state into a second
      state buffer (the rollback cache is armed by reference, so nothing is copied);
      per attention layer: the block-causal SDPA over offset+16 keys with the append of the
-     block's 16 K/V rows at the cache offset fused in;
+     block's 16 K/V rows at the cache offset fused in (dense caches, or paged pools when
+     ``StackConfig.page_size`` is set);
   2. acceptance length / commit count on the device (no host round trip);
   3. rollback: ONE batched tape-replay launch for all GatedDelta layers that reads the
      commit count from device memory and leaves a fully accepted block alone; the KV
@@ -46,6 +47,7 @@ class StackConfig:
     D: int = 256
     context: int = 32768           # L0: cached tokens before the first step
     max_steps: int = 64            # sizes the KV capacity
+    page_size: int = 0             # 0: dense KV caches; otherwise paged pools with pages of this many keys
 
     @property
     def capacity(self) -> int:
@@ -97,6 +99,19 @@ class HybridVerifyStack:
                     v_new=randn(1, cfg.Hkv, T, cfg.D).to(bf), k_cache=kc, v_cache=vc,
                     out=torch.empty(1, cfg.Hq, T, cfg.D, dtype=bf, device=device),
                     lse=torch.empty(1, cfg.Hq, T, dtype=torch.float32, device=device))
+                if cfg.page_size:
+                    # the same keys in a pool [pages, Hkv, page_size, D] under a shuffled page table
+                    P = cfg.page_size
+                    pages = (cfg.capacity + P - 1) // P
+                    perm = torch.randperm(pages, generator=torch.Generator().manual_seed(seed + len(self.attn)))
+                    layer["page_table"] = perm.to(torch.int32).view(1, pages).to(device)
+                    for name, dense in (("k_pool", kc), ("v_pool", vc)):
+                        padded = torch.zeros(cfg.Hkv, pages * P, cfg.D, dtype=bf, device=device)
+                        padded[:, : cfg.capacity] = dense[0]
+                        pool = torch.empty(pages, cfg.Hkv, P, cfg.D, dtype=bf, device=device)
+                        pool[perm.to(device)] = padded.view(cfg.Hkv, pages, P, cfg.D).transpose(0, 1)
+                        layer[name] = pool
+                    del layer["k_cache"], layer["v_cache"]
                 self.attn.append(layer)
         self.scale = 1.0 / (cfg.D ** 0.5)
         n_max = cfg.capacity
@@ -143,6 +158,15 @@ class HybridVerifyStack:
                 l = self.attn[ai]; ai += 1
                 hs = cfg.capacity * cfg.D
                 note("sdpa")
+                if cfg.page_size:
+                    kp = l["k_pool"]
+                    rc = lib.dflash_sdpa_block_causal_paged(
+                        st, _p(l["q"]), _p(kp), _p(l["v_pool"]), _p(l["page_table"]), l["page_table"].shape[1], cfg.page_size,
+                        kp.shape[0], kp.stride(0), kp.stride(1), _p(l["k_new"]), _p(l["v_new"]), _p(l["out"]), _p(l["lse"]),
+                        _lib.BF16, self.scale, 1, cfg.Hq, cfg.Hkv, T, self.n_max, cfg.D, _p(self.offset), _p(self.workspace),
+                        self.workspace.numel())
+                    _lib.check(rc, "sdpa_block_causal_paged")
+                    continue
                 rc = lib.dflash_sdpa_block_causal_append(
                     st, _p(l["q"]), _p(l["k_cache"]), _p(l["v_cache"]), _p(l["k_new"]), _p(l["v_new"]), _p(l["out"]),
                     _p(l["lse"]), _lib.BF16, self.scale, 1, cfg.Hq, cfg.Hkv, T, self.n_max, cfg.D, cfg.Hkv * hs, hs,

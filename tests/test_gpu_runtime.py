@@ -349,3 +349,32 @@ def test_verify_stack_steps_match_oracle_and_fused_accept(gpu_lib):
             ow, _ = O.sdpa_block_causal(host(la["q"]), host(la["k_cache"])[:, :, :n_keys], host(la["v_cache"])[:, :, :n_keys],
                                         a.scale)
             np.testing.assert_allclose(host(la["out"]), ow, rtol=2e-2, atol=2e-2)
+
+
+def test_verify_stack_paged_equals_dense(gpu_lib):
+    """The verify-step driver with paged K/V pools gives the bytes of the dense driver, step after step,
+    and the appended rows sit in the pages the table names."""
+    import torch
+    from swiftlm_amd.verify_step import HybridVerifyStack, StackConfig
+
+    kw = dict(n_layers=8, attn_every=4, block=16, Hk=2, Hv=4, Dk=128, Dv=32, Hq=4, Hkv=2, D=128, context=150, max_steps=6)
+    dense = HybridVerifyStack(StackConfig(**kw), seed=3)
+    paged = HybridVerifyStack(StackConfig(page_size=32, **kw), seed=3)
+    offset = kw["context"]
+    for step, cc in enumerate([3, 16, 1, 9, 5]):
+        for st in (dense, paged):
+            st.set_acceptance(st.phase, cc, seed=step)
+            st.enqueue_step()
+        torch.cuda.synchronize()
+        offset += cc
+        assert int(dense.offset) == int(paged.offset) == offset
+        assert dense.accept.tolist() == paged.accept.tolist()
+        for ld, lp in zip(dense.attn, paged.attn):
+            assert torch.equal(ld["out"], lp["out"]) and torch.equal(ld["lse"], lp["lse"])
+            n_keys = offset - cc + 16                       # rows the step left in the cache (commit or not, all 16 were stored)
+            tb = lp["page_table"][0].cpu().numpy()
+            gathered = O.gather_pages(host(lp["k_pool"]), tb[None], n_keys)
+            assert np.array_equal(gathered, host(ld["k_cache"])[:, :, :n_keys])
+        for ld, lp in zip(dense.gdn, paged.gdn):
+            assert torch.equal(ld["state"][dense.phase], lp["state"][paged.phase])
+
