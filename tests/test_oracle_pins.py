@@ -563,3 +563,27 @@ def test_gdn_finish_against_library_forms():
     np.testing.assert_allclose(np.sqrt((unit ** 2).mean(-1)), 1.0, rtol=1e-12)
     np.testing.assert_allclose(out, unit * w * expit(z), rtol=1e-12)
     np.testing.assert_allclose(O.gdn_finish(y, z, w, 1e-6, "silu"), O.gdn_finish(y, z, w, 1e-6) * z, rtol=1e-12)
+
+
+def test_page_gather_scatter_brute_force():
+    """gather_pages against an element-by-element loop over the page table, scatter_pages as its inverse,
+    and the attention on a gathered cache equal to the attention on the dense one."""
+    rng = np.random.default_rng(11)
+    B, Hk, N, D, P, pages = 2, 3, 75, 4, 32, 9
+    dense = rng.standard_normal((B, Hk, N, D)).astype(np.float32)
+    table = np.array([[7, 2, 5], [0, 8, 3]])
+    pool = O.scatter_pages(dense, table, pages, P, fill=-1.0)
+    for b in range(B):
+        for n in range(N):
+            assert np.array_equal(pool[table[b, n // P], :, n % P], dense[b, :, n])
+    untouched = np.ones(pages, bool)
+    untouched[table.ravel()] = False
+    assert np.all(pool[untouched] == -1.0)                       # pages nobody maps keep the fill
+    assert np.all(pool[table[0, 2], :, N - 2 * P:] == -1.0)      # and so does the unused end of a last page
+    got = O.gather_pages(pool, table, N)
+    assert got.shape == dense.shape and np.array_equal(got, dense)
+    assert np.array_equal(O.gather_pages(pool, table, 40), dense[:, :, :40])
+    q = rng.standard_normal((B, 6, 16, D)).astype(np.float32)
+    o1, l1 = O.sdpa_block_causal(q, dense, dense[::-1].copy(), 0.5)
+    o2, l2 = O.sdpa_block_causal(q, got, O.gather_pages(O.scatter_pages(dense[::-1].copy(), table, pages, P), table, N), 0.5)
+    assert np.array_equal(o1, o2) and np.array_equal(l1, l2)
