@@ -132,7 +132,7 @@ typedef __attribute__((ext_vector_type(8))) short s16x8_t;
 __device__ __forceinline__ void async_load_16B(const unsigned char* gbase, uint32_t goff, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
-                 : "v"(goff), "s"(gbase), "s"(lds_base)
+                 : "v"(goff), "s"(gbase), "s"(__builtin_amdgcn_readfirstlane(lds_base))
                  : "memory", "m0");
 }
 
@@ -148,7 +148,7 @@ __device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char*
 __device__ __forceinline__ void async_load_16B_addr(const unsigned char* gptr, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                  :
-                 : "v"((uint64_t)gptr), "s"(lds_base)
+                 : "v"((uint64_t)gptr), "s"(__builtin_amdgcn_readfirstlane(lds_base))
                  : "memory", "m0");
 }
 
@@ -619,10 +619,18 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
             const float alpha = (bump && m_run != -INFINITY) ? fast_exp2(m_run - m_pending) : 1.f;
             if (bump) m_run = m_pending;
             l_run *= alpha;
+            // The accumulators live in AGPRs inside the loop and this multiply needs them in VGPRs.  Pinning them
+            // to AGPRs on both sides of the multiply makes the compiler copy them HERE; without the pins it
+            // refreshed a VGPR copy of all of them at the end of every loop iteration (128 v_accvgpr_read that
+            // wait for the last MFMA: 0.3 us per tile).
+#pragma unroll
+            for (int i = 0; i < DB; ++i) asm volatile("" : "+a"(oacc[i]));
 #pragma unroll
             for (int i = 0; i < DB; ++i)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
+#pragma unroll
+            for (int i = 0; i < DB; ++i) asm volatile("" : "+a"(oacc[i]));
             ++t;                                   // x already holds tile t+1's scores
         }
     }
