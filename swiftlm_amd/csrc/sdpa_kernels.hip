@@ -84,7 +84,7 @@ struct SdpaArgs {
     const uint16_t* v_new;
     uint16_t* k_cache;       // where the fused append stores those rows (== k, v), or null
     uint16_t* v_cache;
-    uint16_t* part_o;   // [S, B*Hq*16, D]  unnormalised partial O in the input type (DFlashKernels.swift:647)
+    uint16_t* part_o;   // [S, B*Hq*16, D]  partial O / l in the input type (DFlashKernels.swift:647 stores it unnormalised)
     float* part_m;   // [B*Hq*16, S]   running max, log2 units
     float* part_l;   // [B*Hq*16, S]   sum of exp2
     const int32_t* kv_len_dev;
@@ -647,6 +647,11 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
         A.part_l[row_id * A.S + split] = l_tot;
     }
     if (wave_active) {
+        // Partial rows are stored NORMALISED (O / l): the reference keeps them unnormalised in the input type
+        // (DFlashKernels.swift:647) with exponents taken against each block's exact maximum; here the exponent
+        // reference may lag the maximum by 2^kRescaleLog2 and a split spans hundreds of keys, so the raw sums can
+        // pass the largest f16 value.  The combine kernel weights by l accordingly.
+        const float inv_l = l_tot > 0.f ? 1.f / l_tot : 0.f;
         // Rows are rounded to the input type first and staged as such: lane (c, h) holds 4 consecutive
         // channels of row c per accumulator quad (8 bytes); the row pitch of D*2 + 16 bytes keeps the
         // 8-byte writes and the 16-byte reads below spread over the banks.
@@ -655,7 +660,8 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
         for (int i = 0; i < DB; ++i)
 #pragma unroll
             for (int v4 = 0; v4 < 4; ++v4) {
-                const f32x4_t o4 = {oacc[i][4 * v4], oacc[i][4 * v4 + 1], oacc[i][4 * v4 + 2], oacc[i][4 * v4 + 3]};
+                const f32x4_t o4 = {oacc[i][4 * v4] * inv_l, oacc[i][4 * v4 + 1] * inv_l, oacc[i][4 * v4 + 2] * inv_l,
+                                    oacc[i][4 * v4 + 3] * inv_l};
                 const u32x2_t pk = __builtin_bit_cast(u32x2_t, Tag::pack4(o4));      // hardware round-to-nearest-even
                 *reinterpret_cast<u32x2_t*>(os + c * L::EROW + (32 * i + 8 * v4 + 4 * h) * 2) = pk;
             }
@@ -717,9 +723,9 @@ __global__ __launch_bounds__(kSdpaThreads) void sdpa_combine_kernel(CombineArgs 
     float lsum = 0.f;
     for (int s = tid; s < A.S; s += kSdpaThreads) {
         const float m = pm[s];
-        const float w = m == -INFINITY ? 0.f : fast_exp2(m - mx);
+        const float w = m == -INFINITY ? 0.f : fast_exp2(m - mx) * pl[s];   // the partial rows are O / l: weight by l
         w_s[s] = w;
-        lsum += w * pl[s];
+        lsum += w;
     }
     for (int o = 32; o >= 1; o >>= 1) lsum += __shfl_xor(lsum, o);
     if ((tid & 63) == 0) red_s[tid >> 6] = lsum;

@@ -243,3 +243,25 @@ def test_sdpa_fused_append_ragged(gpu_lib):
     got = K.batched_sdpa_2pass_append(q, kc, vc, k_new, v_new, 1.0 / 16, cap, cache_len=cache_len)
     assert torch.equal(got, want)
     assert torch.equal(kc, k) and torch.equal(vc, v)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+def test_sdpa_partial_rows_do_not_overflow_f16(gpu_lib, dtype):
+    """Scores that rise by just under the lazy-rescale threshold after the first tile make the
+    unnormalised partial sums of a split large (2^7.9 x 224 keys x |V| = 2e5 here): the partial rows
+    are stored normalised, so an f16 run still returns the exact answer (every V row is 4)."""
+    from swiftlm_amd import DFlashKernels as K
+
+    B, Hq, Hk, D, L = 1, 8, 1, 128, 32768
+    N = L + 16
+    q = torch.zeros(B, Hq, 16, D, dtype=dtype, device="cuda")
+    q[..., 0] = 1.0
+    k = torch.zeros(B, Hk, N, D, dtype=dtype, device="cuda")
+    k[:, :, 32:, 0] = 7.9 / 1.4426950408889634
+    v = torch.full((B, Hk, N, D), 4.0, dtype=dtype, device="cuda")
+    out, lse = K.batched_sdpa_2pass(q, k, v, 1.0, return_lse=True)
+    want, want_lse = torch_reference(q, k, v, 1.0)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())
+    np.testing.assert_allclose(host(out), 4.0, rtol=1e-2)
+    np.testing.assert_allclose(host(lse), host(want_lse), **LSE_TOL)
