@@ -687,6 +687,450 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
     }
 }
 
+// ---------------------------------------------------------------------------
+// Producer/consumer form of the partial kernel (dense and fused-append calls).
+//
+// A wave that issues HBM -> LDS loads is held at each load until the memory pipeline takes it; in the
+// streaming steady state that is most of a tile's transfer time, and a wave that is held cannot feed
+// its MFMAs.  Here waves 0..3 only compute and waves 4..5 only request tiles and wait for them, so the
+// holds fall on waves with nothing else to do.  Six waves put two on a SIMD, i.e. 256 registers per
+// wave: Q (64 registers per lane in the kernel above) stays in LDS and is read per k-step like K.
+//
+// LDS: Q [128 rows] | K ring, kPcSlots tiles | V ring, kPcSlots tiles.  K and V advance separately because
+// the scores run one tile ahead of the PV product: iteration t needs V(t) and K(t+1) ("group t").
+// Producers: request Q + K(t0), group t0, group t0+1; then per iteration t: wait for group t, barrier,
+// request group t+2 (V(t+2) into the slot of V(t-1), K(t+3) into the slot of K(t), both free after
+// the barrier).  One barrier per iteration, shared by all six waves.
+// ---------------------------------------------------------------------------
+constexpr int kPcThreads = 384;
+constexpr int kPcSlots = 3;
+
+template <int D> struct PcLds {
+    static constexpr int ROWB = D * 2;
+    static constexpr int CPR = D / 8;
+    static constexpr int RPI = 64 / CPR;                     // rows per 1 KB load instruction
+    static constexpr int KT = kBN * ROWB;                    // bytes of one K (or V) tile
+    static constexpr int Q_BYTES = 4 * 32 * ROWB;            // 32 query rows per compute wave
+    static constexpr int K_RING = Q_BYTES;
+    static constexpr int V_RING = Q_BYTES + kPcSlots * KT;
+    static constexpr int LPP = (kBN / RPI) / 2;              // load instructions per producer wave per K (or V) tile
+    static constexpr int QPP = (128 / RPI) / 2;              // ... for Q
+    static constexpr int EROW = D * 2 + 16;
+    static constexpr int EPI = 4 * 32 * EROW;
+    static constexpr int RING_END = Q_BYTES + 2 * kPcSlots * KT;
+    static constexpr int BYTES = RING_END > EPI ? RING_END : EPI;
+};
+
+template <typename Tag, int D>
+__global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs A) {
+    typedef typename Tag::vec8 vec8;
+    typedef PcLds<D> L;
+    constexpr int KSTEPS = D / 16;
+    constexpr int DB = D / 32;
+    static_assert(2 * L::LPP + L::QPP <= 63 && 4 * L::LPP <= 63, "vmcnt is a 6-bit counter");
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const uint32_t smem_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool producer = wave >= 4;
+    const int c = lane & 31, h = lane >> 5;
+    const int split = blockIdx.x;
+    const int hk = blockIdx.y / A.groups_per_kv;
+    const int hg0 = (blockIdx.y % A.groups_per_kv) * kHeadsPerWG;
+    const int b = blockIdx.z;
+    const int hcount = (A.G - hg0) < kHeadsPerWG ? (A.G - hg0) : kHeadsPerWG;
+
+    int Nb = A.kv_len_dev ? A.kv_len_dev[b] + A.len_bias : A.N;
+    Nb = Nb < kM ? kM : (Nb > A.N ? A.N : Nb);
+    const int nt = (Nb + kBN - 1) / kBN;
+    const int t_begin = (int)(((long)split * nt) / A.S);
+    const int t_end = (int)(((long)(split + 1) * nt) / A.S);
+    const int t_last = t_end - 1;
+
+    const int cw = producer ? 0 : wave;                      // compute wave index (producers: unused)
+    const int head_in_group = 2 * cw + (c >> 4);
+    const bool row_valid = !producer && head_in_group < hcount;
+    const bool wave_active = !producer && 2 * cw < hcount;
+    const int hq = hk * A.G + hg0 + head_in_group;
+    const int qi = c & 15;
+    const size_t row_id = ((size_t)b * A.Hq + hq) * kM + qi;
+
+    const size_t head_off = ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
+    const unsigned char* kbase = reinterpret_cast<const unsigned char*>(A.k) + head_off;
+    const unsigned char* vbase = reinterpret_cast<const unsigned char*>(A.v) + head_off;
+    const bool fused = A.k_new != nullptr;
+    const int cache_rows = fused ? Nb - kM : Nb;
+    const unsigned char* knew = reinterpret_cast<const unsigned char*>(A.k_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
+    const unsigned char* vnew = reinterpret_cast<const unsigned char*>(A.v_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
+    if (fused && A.k_cache && split == 0 && hg0 == 0) {
+        const size_t head = head_off + (size_t)cache_rows * L::ROWB;
+        u32x4_t* kd = reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.k_cache) + head);
+        u32x4_t* vd = reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.v_cache) + head);
+        const u32x4_t* ksrc = reinterpret_cast<const u32x4_t*>(knew);
+        const u32x4_t* vsrc = reinterpret_cast<const u32x4_t*>(vnew);
+        for (int i = tid; i < kM * L::CPR; i += kPcThreads) { kd[i] = ksrc[i]; vd[i] = vsrc[i]; }
+    }
+
+    if (t_begin >= t_end) {   // empty split: tell the combine kernel to ignore it
+        if (row_valid && h == 0) {
+            A.part_m[row_id * A.S + split] = -INFINITY;
+            A.part_l[row_id * A.S + split] = 0.f;
+        }
+        return;
+    }
+
+    // =========================== producers ===========================
+    if (producer) {
+        const int pw = wave - 4;
+        const int ld_rsub = lane / L::CPR, ld_pos = lane % L::CPR;
+        // instruction j of this producer covers rows (2*j + pw) * RPI .. + RPI - 1 of a tile (or of Q)
+        auto issue_rows = [&](const unsigned char* base, bool k_swizzle, int t, uint32_t lds_tile, bool is_k) {
+            const int key0 = t * kBN;
+            if (key0 + kBN <= cache_rows) {              // uniform: whole tile comes from the cache
+                const unsigned char* tp = uniform_ptr(base + (size_t)key0 * L::ROWB);
+#pragma unroll
+                for (int j = 0; j < L::LPP; ++j) {
+                    const int rg = (2 * j + pw) * L::RPI;
+                    const int row = rg + ld_rsub;
+                    const uint32_t sw = k_swizzle ? (uint32_t)((ld_pos ^ (row & 15)) * 16) : (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
+                    async_load_16B(tp, (uint32_t)row * L::ROWB + sw, lds_tile + rg * L::ROWB);
+                }
+            } else {
+                // Tail tile: rows past the end re-read the last key (masked later); with a fused append the
+                // block's own 16 rows are taken from k_new / v_new instead of the cache.
+#pragma unroll
+                for (int j = 0; j < L::LPP; ++j) {
+                    const int rg = (2 * j + pw) * L::RPI;
+                    const int row = rg + ld_rsub;
+                    int key = key0 + row;
+                    key = key < Nb ? key : Nb - 1;
+                    const uint32_t sw = k_swizzle ? (uint32_t)((ld_pos ^ (row & 15)) * 16) : (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
+                    const unsigned char* nw = is_k ? knew : vnew;
+                    const unsigned char* src = key < cache_rows ? base + (size_t)key * L::ROWB : nw + (size_t)(key - cache_rows) * L::ROWB;
+                    async_load_16B_addr(src + sw, lds_tile + rg * L::ROWB);
+                }
+            }
+        };
+        auto issue_k = [&](int t) {
+            if (t < t_end) issue_rows(kbase, true, t, smem_lds + L::K_RING + ((t - t_begin) % kPcSlots) * L::KT, true);
+        };
+        auto issue_v = [&](int t) {
+            if (t < t_end) issue_rows(vbase, false, t, smem_lds + L::V_RING + ((t - t_begin) % kPcSlots) * L::KT, false);
+        };
+        // loads of group t still outstanding when one waits for the group before it
+        auto group_loads = [&](int t) { return (t < t_end ? L::LPP : 0) + (t + 1 < t_end ? L::LPP : 0); };
+
+        // Q: the 32 rows of compute wave w (heads 2w, 2w+1 of the group), swizzled like a K tile, at w * 32 rows.
+        // An absent head re-reads the group's first head (its rows are never stored).
+        {
+            const unsigned char* qb = reinterpret_cast<const unsigned char*>(A.q) + ((size_t)b * A.Hq + hk * A.G + hg0) * kM * L::ROWB;
+#pragma unroll
+            for (int j = 0; j < L::QPP; ++j) {
+                const int row = (2 * j + pw) * L::RPI + ld_rsub;           // 0..127 over the four compute waves
+                const int head = (row >> 4) < hcount ? (row >> 4) : 0;
+                async_load_16B_addr(qb + (size_t)(head * kM + (row & 15)) * L::ROWB + ((ld_pos ^ (row & 15)) * 16),
+                                    smem_lds + (2 * j + pw) * L::RPI * L::ROWB);
+            }
+        }
+        issue_k(t_begin);
+        issue_v(t_begin); issue_k(t_begin + 1);            // group t_begin
+        issue_v(t_begin + 1); issue_k(t_begin + 2);        // group t_begin + 1
+        {
+            const int later = group_loads(t_begin) + group_loads(t_begin + 1);     // 0 .. 4 * LPP
+            if (later >= 4 * L::LPP) wait_vmcnt<4 * L::LPP>();
+            else if (later >= 3 * L::LPP) wait_vmcnt<3 * L::LPP>();
+            else if (later >= 2 * L::LPP) wait_vmcnt<2 * L::LPP>();
+            else if (later >= L::LPP) wait_vmcnt<L::LPP>();
+            else wait_vmcnt<0>();
+        }
+        __builtin_amdgcn_s_barrier();                       // Q and K(t_begin) are in LDS
+        for (int t = t_begin; t <= t_last; ++t) {
+            const int later = group_loads(t + 1);
+            if (later >= 2 * L::LPP) wait_vmcnt<2 * L::LPP>();
+            else if (later >= L::LPP) wait_vmcnt<L::LPP>();
+            else wait_vmcnt<0>();
+            __builtin_amdgcn_s_barrier();                   // group t is in LDS; iteration t-1 is over for every wave
+            issue_v(t + 2); issue_k(t + 3);                 // group t + 2, into the slots iteration t-1 released
+        }
+        return;
+    }
+
+    // =========================== compute waves ===========================
+    const int k_rd = c * L::ROWB;
+    const int k_sw = c & 15;
+    const int tj = (lane & 15) >> 2, tq = lane & 3;
+    const int tg = lane >> 4;
+    const int v_rd = (4 * (tg >> 1) + tj) * L::ROWB + (tq & 1) * 8;
+    const int v_piece = 2 * (tg & 1) + (tq >> 1);
+    const int v_sw = 4 * tj;
+    const unsigned char* q_rows = smem + cw * 32 * L::ROWB;
+
+    auto k_slot = [&](int t) -> const unsigned char* { return smem + L::K_RING + ((t - t_begin) % kPcSlots) * L::KT; };
+    auto v_slot = [&](int t) -> const unsigned char* { return smem + L::V_RING + ((t - t_begin) % kPcSlots) * L::KT; };
+    // Operand offsets inside a tile.  The XOR swizzles only touch the low bits of the piece index, so a handful of
+    // per-lane offsets plus compile-time constants (folded into the ds_read offset field) cover every k-step:
+    //   K, Q: piece (2s+h) ^ (c & 15) = 16 * (s >> 3) + ((2 * (s & 7) + h) ^ (c & 15))
+    //   V:    piece (4i + v_piece) ^ (4 tj) = 16 * (i >> 2) + 4 * ((i & 3) ^ tj) + v_piece
+    uint32_t koff[8], voff[4];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) koff[j] = (uint32_t)(k_rd + (((2 * j + h) ^ k_sw) & (L::CPR - 1)) * 16);
+#pragma unroll
+    for (int m = 0; m < 4; ++m) voff[m] = (uint32_t)(v_rd + v_piece * 16 + ((m ^ tj) * 64));
+    (void)v_sw;
+    auto load_k = [&](const unsigned char* ks, int s) -> vec8 {
+        return *reinterpret_cast<const vec8*>(ks + koff[s & 7] + 256 * (s >> 3));
+    };
+    auto load_q = [&](int s) -> vec8 {
+        return *reinterpret_cast<const vec8*>(q_rows + koff[s & 7] + 256 * (s >> 3));
+    };
+    auto load_v = [&](const unsigned char* vs, int s) -> vec8 {
+        const int i = s % DB, ksub = s / DB;
+        const unsigned char* p = vs + voff[i & 3] + 256 * (i >> 2);
+        const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4_t*)(p + (16 * ksub) * L::ROWB));
+        const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4_t*)(p + (16 * ksub + 8) * L::ROWB));
+        return __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+    // operand reads run this many MFMA steps ahead; 2 at D = 256 keeps the wave inside its 256 registers without spills
+    constexpr int kAhead = D == 256 ? 2 : 4;
+
+    f32x16_t oacc[DB];
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) oacc[i][v] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+    float x[16];
+    vec8 pb[2];
+    f32x16_t sacc, sacc1;
+    float m_pending = -INFINITY;
+
+    auto qk_tile = [&](int t) {
+        const unsigned char* ks = k_slot(t);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) { sacc[v] = 0.f; sacc1[v] = 0.f; }
+        vec8 ka[KSTEPS], qa[KSTEPS];
+#pragma unroll
+        for (int s = 0; s < kAhead; ++s) { ka[s] = load_k(ks, s); qa[s] = load_q(s); }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KSTEPS; s += 2) {
+            if (s + kAhead < KSTEPS) {
+                ka[s + kAhead] = load_k(ks, s + kAhead); ka[s + kAhead + 1] = load_k(ks, s + kAhead + 1);
+                qa[s + kAhead] = load_q(s + kAhead); qa[s + kAhead + 1] = load_q(s + kAhead + 1);
+            }
+            sacc = Tag::mfma(ka[s], qa[s], sacc);
+            sacc1 = Tag::mfma(ka[s + 1], qa[s + 1], sacc1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto exp_qk = [&](int t) {
+        const unsigned char* ks = k_slot(t + 1);
+        const float m_safe = m_run == -INFINITY ? 0.f : m_run;
+        float psum = 0.f;
+        f32x8_t p0, p1;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) { sacc[v] = 0.f; sacc1[v] = 0.f; }
+        vec8 ka[KSTEPS], qa[KSTEPS];
+#pragma unroll
+        for (int s = 0; s < kAhead; ++s) { ka[s] = load_k(ks, s); qa[s] = load_q(s); }
+        __builtin_amdgcn_sched_barrier(0);
+        constexpr int PAIRS = KSTEPS / 2;
+        constexpr int EPP = 16 / PAIRS;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; s += 2) {
+            if (s + kAhead < KSTEPS) {
+                ka[s + kAhead] = load_k(ks, s + kAhead); ka[s + kAhead + 1] = load_k(ks, s + kAhead + 1);
+                qa[s + kAhead] = load_q(s + kAhead); qa[s + kAhead + 1] = load_q(s + kAhead + 1);
+            }
+            sacc = Tag::mfma(ka[s], qa[s], sacc);
+            sacc1 = Tag::mfma(ka[s + 1], qa[s + 1], sacc1);
+            const int pr = s / 2;
+#pragma unroll
+            for (int e = pr * EPP; e < (pr + 1) * EPP; ++e) {
+                const float pe = fast_exp2(x[e] - m_safe);
+                psum += pe;
+                if (e < 8) p0[e] = pe; else p1[e - 8] = pe;
+            }
+            if ((pr + 1) * EPP == 8) pb[0] = Tag::pack(p0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        pb[1] = Tag::pack(p1);
+        l_run += psum;
+    };
+    auto pv_scale = [&](int t) -> float {
+        const unsigned char* vs = v_slot(t);
+        vec8 va[KSTEPS];
+#pragma unroll
+        for (int s = 0; s < kAhead; ++s) va[s] = load_v(vs, s);
+        __builtin_amdgcn_sched_barrier(0);
+        float mloc = -INFINITY;
+        constexpr int EPS = 16 / KSTEPS;
+        constexpr int LAG = 2;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+            if (s + kAhead < KSTEPS) va[s + kAhead] = load_v(vs, s + kAhead);
+            oacc[s % DB] = Tag::mfma(va[s], pb[s / DB], oacc[s % DB]);
+            if (s >= LAG) {
+#pragma unroll
+                for (int e = (s - LAG) * EPS; e < (s - LAG + 1) * EPS; ++e) {
+                    x[e] = (sacc[e] + sacc1[e]) * A.scale_log2;
+                    mloc = fmaxf(mloc, x[e]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int e = (KSTEPS - LAG) * EPS; e < 16; ++e) {
+            x[e] = (sacc[e] + sacc1[e]) * A.scale_log2;
+            mloc = fmaxf(mloc, x[e]);
+        }
+        return mloc;
+    };
+    auto mask_and_max = [&](int t, float mloc) -> float {
+        const int key0 = t * kBN;
+        if ((key0 + kBN) > (Nb - kM)) {            // uniform: the tile reaches into the block's own keys
+            const int last_visible = Nb - kM + qi;
+            mloc = -INFINITY;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int key = key0 + 8 * (v >> 2) + 4 * h + (v & 3);
+                x[v] = key <= last_visible ? x[v] : -INFINITY;
+                mloc = fmaxf(mloc, x[v]);
+            }
+        }
+        return fmaxf(mloc, __shfl_xor(mloc, 32));
+    };
+    auto accept_max = [&](float ml) -> bool {
+        const bool bump = ml > m_run + kRescaleLog2;
+        if (__builtin_amdgcn_ballot_w64(bump && m_run != -INFINITY) != 0) {
+            m_pending = ml;
+            return false;
+        }
+        if (bump) m_run = ml;
+        return true;
+    };
+    auto exp_tile = [&]() {
+        const float m_safe = m_run == -INFINITY ? 0.f : m_run;
+        float psum = 0.f;
+        f32x8_t p0, p1;
+#pragma unroll
+        for (int v = 0; v < 8; ++v) {
+            p0[v] = fast_exp2(x[v] - m_safe);
+            p1[v] = fast_exp2(x[v + 8] - m_safe);
+            psum += p0[v] + p1[v];
+        }
+        l_run += psum;
+        pb[0] = Tag::pack(p0);
+        pb[1] = Tag::pack(p1);
+    };
+    auto pv_tile = [&](int t) {
+        const unsigned char* vs = v_slot(t);
+        vec8 va[KSTEPS];
+#pragma unroll
+        for (int s = 0; s < kAhead; ++s) va[s] = load_v(vs, s);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+            if (s + kAhead < KSTEPS) va[s + kAhead] = load_v(vs, s + kAhead);
+            oacc[s % DB] = Tag::mfma(va[s], pb[s / DB], oacc[s % DB]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    __builtin_amdgcn_s_barrier();                   // Q and K(t_begin) are in LDS
+    if (wave_active) {
+        qk_tile(t_begin);
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            x[v] = (sacc[v] + sacc1[v]) * A.scale_log2;
+            mloc = fmaxf(mloc, x[v]);
+        }
+        accept_max(mask_and_max(t_begin, mloc));
+    }
+    int t = t_begin;
+    while (t < t_last) {
+        bool jumped = false;
+        for (; t < t_last; ++t) {
+            __builtin_amdgcn_s_barrier();           // V(t) and K(t+1) are in LDS; everyone is done with iteration t-1
+            if (wave_active) {
+                exp_qk(t);
+                const float mloc = pv_scale(t);
+                if (!accept_max(mask_and_max(t + 1, mloc))) {
+                    jumped = true;
+                    break;
+                }
+            }
+        }
+        if (jumped) {
+            const bool bump = m_pending > m_run + kRescaleLog2;
+            const float alpha = (bump && m_run != -INFINITY) ? fast_exp2(m_run - m_pending) : 1.f;
+            if (bump) m_run = m_pending;
+            l_run *= alpha;
+            // (no AGPR pins here: with 256 registers per wave and no "a" constraint in the function the compiler
+            //  keeps every MFMA accumulator in VGPRs, so this multiply works on them in place)
+#pragma unroll
+            for (int i = 0; i < DB; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
+            ++t;
+        }
+    }
+    __builtin_amdgcn_s_barrier();                   // V(t_last) is in LDS
+    if (wave_active) {
+        exp_tile();
+        pv_tile(t_last);
+    }
+    // The epilogue stages rows in the first EPI bytes of LDS (Q and the head of the K ring): nobody reads those
+    // after the barrier above (the last scores were taken in iteration t_last - 1), and every load has landed
+    // (the producers' last wait was vmcnt(0)).
+    static_assert(L::EPI <= L::V_RING, "the epilogue staging must stay clear of the V ring");
+
+    // ---- epilogue: partial statistics and O rows (as in the kernel above) ----
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (row_valid && h == 0) {
+        A.part_m[row_id * A.S + split] = m_run;
+        A.part_l[row_id * A.S + split] = l_tot;
+    }
+    if (wave_active) {
+        const float inv_l = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        unsigned char* os = smem + cw * 32 * L::EROW;
+#pragma unroll
+        for (int i = 0; i < DB; ++i)
+#pragma unroll
+            for (int v4 = 0; v4 < 4; ++v4) {
+                const f32x4_t o4 = {oacc[i][4 * v4] * inv_l, oacc[i][4 * v4 + 1] * inv_l, oacc[i][4 * v4 + 2] * inv_l,
+                                    oacc[i][4 * v4 + 3] * inv_l};
+                const u32x2_t pk = __builtin_bit_cast(u32x2_t, Tag::pack4(o4));
+                *reinterpret_cast<u32x2_t*>(os + c * L::EROW + (32 * i + 8 * v4 + 4 * h) * 2) = pk;
+            }
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        const int rows = (hcount - 2 * cw) >= 2 ? 32 : 16;
+        const size_t rid0 = ((size_t)b * A.Hq + hk * A.G + hg0 + 2 * cw) * kM;
+        constexpr int PER_ROW = D / 8;
+        constexpr int RPP = 64 / PER_ROW;
+        const int rsub = lane / PER_ROW, d = (lane % PER_ROW) * 8;
+        uint16_t* dst = A.part_o + ((size_t)split * A.rows_total + rid0) * D + d;
+#pragma unroll
+        for (int r0 = 0; r0 < 32; r0 += 8 * RPP) {
+            u32x4_t o[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) o[u] = *reinterpret_cast<const u32x4_t*>(os + (r0 + u * RPP + rsub) * L::EROW + d * 2);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int r = r0 + u * RPP + rsub;
+                if (r < rows) *reinterpret_cast<u32x4_t*>(dst + (size_t)r * D) = o[u];
+            }
+        }
+    }
+}
+
 // One workgroup per output row (b, hq, i): merges the S partials.
 struct CombineArgs {
     const uint16_t* part_o;
@@ -801,6 +1245,33 @@ static size_t ws_layout(int B, int Hq, int S, int D, size_t* off_m, size_t* off_
     *off_l = o;
     o += rows * S * sizeof(float);
     return (o + 255) & ~(size_t)255;
+}
+
+static bool use_producer_kernel() {
+    static const bool on = [] { const char* e = getenv("DFLASH_SDPA_PRODUCERS"); return !(e && e[0] == '0'); }();
+    return on;
+}
+
+template <typename Tag, int D>
+static int launch_sdpa_pc(hipStream_t st, const SdpaArgs& A, const CombineArgs& C, int B) {
+    typedef PcLds<D> L;
+    static_assert(L::BYTES <= 160 * 1024, "Q and the tile rings must fit the 160 KB LDS of a gfx950 CU");
+    auto kern = sdpa_partial_pc_kernel<Tag, D>;
+    static const hipError_t attr_rc =
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::BYTES);
+    DFLASH_HIP_TRY(attr_rc);
+    dim3 grid(A.S, A.Hk * A.groups_per_kv, B);
+    {
+        LaunchBracket br(DFLASH_KERNEL_SDPA_PARTIAL, st);
+        br.launch(kern, grid, dim3(kPcThreads), L::BYTES, A);
+    }
+    DFLASH_HIP_TRY(hipGetLastError());
+    {
+        LaunchBracket br(DFLASH_KERNEL_SDPA_COMBINE, st);
+        br.launch(sdpa_combine_kernel<Tag, D>, dim3(B * A.Hq * kM), dim3(kSdpaThreads), 0, C);
+    }
+    DFLASH_HIP_TRY(hipGetLastError());
+    return DFLASH_OK;
 }
 
 template <typename Tag, int D, bool MASKED, bool PAGED>
@@ -925,6 +1396,10 @@ static int sdpa_common(void* stream, const void* q, const void* k, const void* v
     if (paged) {
         if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa<Bf16Tag, 256, false, true>(st, A, C, B) : launch_sdpa<Bf16Tag, 128, false, true>(st, A, C, B);
         return D == 256 ? launch_sdpa<F16Tag, 256, false, true>(st, A, C, B) : launch_sdpa<F16Tag, 128, false, true>(st, A, C, B);
+    }
+    if (use_producer_kernel()) {
+        if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa_pc<Bf16Tag, 256>(st, A, C, B) : launch_sdpa_pc<Bf16Tag, 128>(st, A, C, B);
+        return D == 256 ? launch_sdpa_pc<F16Tag, 256>(st, A, C, B) : launch_sdpa_pc<F16Tag, 128>(st, A, C, B);
     }
     if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa<Bf16Tag, 256, false, false>(st, A, C, B) : launch_sdpa<Bf16Tag, 128, false, false>(st, A, C, B);
     return D == 256 ? launch_sdpa<F16Tag, 256, false, false>(st, A, C, B) : launch_sdpa<F16Tag, 128, false, false>(st, A, C, B);
