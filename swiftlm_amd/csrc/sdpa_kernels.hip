@@ -746,9 +746,14 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
     int Nb = A.kv_len_dev ? A.kv_len_dev[b] + A.len_bias : A.N;
     Nb = Nb < kM ? kM : (Nb > A.N ? A.N : Nb);
     const int nt = (Nb + kBN - 1) / kBN;
-    const int t_begin = (int)(((long)split * nt) / A.S);
-    const int t_end = (int)(((long)(split + 1) * nt) / A.S);
+    // Tiles are dealt round-robin: split s takes tiles s, s + S, s + 2S, ...  At any moment the workgroups of a KV
+    // head then read one contiguous stretch of the cache (S neighbouring tiles) instead of S stretches a split
+    // apart, which the memory system serves faster.  Below, t counts this split's own tiles (0 .. t_end-1) and
+    // key_of(t) is the first key of its t-th tile.
+    const int t_begin = 0;
+    const int t_end = split < nt ? (nt - split + A.S - 1) / A.S : 0;
     const int t_last = t_end - 1;
+    auto key_of = [&](int t) { return (split + t * A.S) * kBN; };
 
     const int cw = producer ? 0 : wave;                      // compute wave index (producers: unused)
     const int head_in_group = 2 * cw + (c >> 4);
@@ -788,7 +793,7 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
         const int ld_rsub = lane / L::CPR, ld_pos = lane % L::CPR;
         // instruction j of this producer covers rows (2*j + pw) * RPI .. + RPI - 1 of a tile (or of Q)
         auto issue_rows = [&](const unsigned char* base, bool k_swizzle, int t, uint32_t lds_tile, bool is_k) {
-            const int key0 = t * kBN;
+            const int key0 = key_of(t);
             if (key0 + kBN <= cache_rows) {              // uniform: whole tile comes from the cache
                 const unsigned char* tp = uniform_ptr(base + (size_t)key0 * L::ROWB);
 #pragma unroll
@@ -992,7 +997,7 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
         return mloc;
     };
     auto mask_and_max = [&](int t, float mloc) -> float {
-        const int key0 = t * kBN;
+        const int key0 = key_of(t);
         if ((key0 + kBN) > (Nb - kM)) {            // uniform: the tile reaches into the block's own keys
             const int last_visible = Nb - kM + qi;
             mloc = -INFINITY;
@@ -1247,9 +1252,11 @@ static size_t ws_layout(int B, int Hq, int S, int D, size_t* off_m, size_t* off_
     return (o + 255) & ~(size_t)255;
 }
 
+// DFLASH_SDPA_PRODUCERS=0 selects the single-role kernel for every call (A/B runs, and the tests that compare
+// the paged entry, which always uses that kernel, byte for byte with the dense one).  Read at each call.
 static bool use_producer_kernel() {
-    static const bool on = [] { const char* e = getenv("DFLASH_SDPA_PRODUCERS"); return !(e && e[0] == '0'); }();
-    return on;
+    const char* e = getenv("DFLASH_SDPA_PRODUCERS");
+    return !(e && e[0] == '0');
 }
 
 template <typename Tag, int D>
