@@ -698,7 +698,7 @@ __global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs 
 //
 // LDS: Q [128 rows] | K ring, kPcSlots tiles | V ring, kPcSlots tiles.  K and V advance separately because
 // the scores run one tile ahead of the PV product: iteration t needs V(t) and K(t+1) ("group t").
-// Producers: request Q + K(t0), group t0, group t0+1; then per iteration t: wait for group t, barrier,
+// Producers: request K(t0), group t0, group t0+1 (each compute wave requests its own Q rows meanwhile); then per iteration t: wait for group t, barrier,
 // request group t+2 (V(t+2) into the slot of V(t-1), K(t+3) into the slot of K(t), both free after
 // the barrier).  One barrier per iteration, shared by all six waves.
 // ---------------------------------------------------------------------------
@@ -714,7 +714,7 @@ template <int D> struct PcLds {
     static constexpr int K_RING = Q_BYTES;
     static constexpr int V_RING = Q_BYTES + kPcSlots * KT;
     static constexpr int LPP = (kBN / RPI) / 2;              // load instructions per producer wave per K (or V) tile
-    static constexpr int QPP = (128 / RPI) / 2;              // ... for Q
+    static constexpr int QPW = 32 / RPI;                     // load instructions per compute wave for its Q rows
     static constexpr int EROW = D * 2 + 16;
     static constexpr int EPI = 4 * 32 * EROW;
     static constexpr int RING_END = Q_BYTES + 2 * kPcSlots * KT;
@@ -727,7 +727,7 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
     typedef PcLds<D> L;
     constexpr int KSTEPS = D / 16;
     constexpr int DB = D / 32;
-    static_assert(2 * L::LPP + L::QPP <= 63 && 4 * L::LPP <= 63, "vmcnt is a 6-bit counter");
+    static_assert(4 * L::LPP <= 63 && L::QPW <= 63, "vmcnt is a 6-bit counter");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t smem_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
@@ -828,18 +828,6 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
         // loads of group t still outstanding when one waits for the group before it
         auto group_loads = [&](int t) { return (t < t_end ? L::LPP : 0) + (t + 1 < t_end ? L::LPP : 0); };
 
-        // Q: the 32 rows of compute wave w (heads 2w, 2w+1 of the group), swizzled like a K tile, at w * 32 rows.
-        // An absent head re-reads the group's first head (its rows are never stored).
-        {
-            const unsigned char* qb = reinterpret_cast<const unsigned char*>(A.q) + ((size_t)b * A.Hq + hk * A.G + hg0) * kM * L::ROWB;
-#pragma unroll
-            for (int j = 0; j < L::QPP; ++j) {
-                const int row = (2 * j + pw) * L::RPI + ld_rsub;           // 0..127 over the four compute waves
-                const int head = (row >> 4) < hcount ? (row >> 4) : 0;
-                async_load_16B_addr(qb + (size_t)(head * kM + (row & 15)) * L::ROWB + ((ld_pos ^ (row & 15)) * 16),
-                                    smem_lds + (2 * j + pw) * L::RPI * L::ROWB);
-            }
-        }
         issue_k(t_begin);
         issue_v(t_begin); issue_k(t_begin + 1);            // group t_begin
         issue_v(t_begin + 1); issue_k(t_begin + 2);        // group t_begin + 1
@@ -851,7 +839,7 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
             else if (later >= L::LPP) wait_vmcnt<L::LPP>();
             else wait_vmcnt<0>();
         }
-        __builtin_amdgcn_s_barrier();                       // Q and K(t_begin) are in LDS
+        __builtin_amdgcn_s_barrier();                       // K(t_begin) is in LDS (and each compute wave's Q rows)
         for (int t = t_begin; t <= t_last; ++t) {
             const int later = group_loads(t + 1);
             if (later >= 2 * L::LPP) wait_vmcnt<2 * L::LPP>();
@@ -1047,7 +1035,23 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
         }
     };
 
-    __builtin_amdgcn_s_barrier();                   // Q and K(t_begin) are in LDS
+    // Q: this wave's own 32 rows (heads 2w, 2w+1 of the group), swizzled like a K tile, at w * 32 rows of the Q
+    // area.  Each compute wave requests its own rows while the producers are already requesting K and V; nobody
+    // else reads them, so the wave's own wait is all the synchronisation they need.  An absent head re-reads the
+    // group's first head (its rows are never stored).
+    if (wave_active) {
+        const int ld_rsub = lane / L::CPR, ld_pos = lane % L::CPR;
+        const unsigned char* qb = reinterpret_cast<const unsigned char*>(A.q) + ((size_t)b * A.Hq + hk * A.G + hg0) * kM * L::ROWB;
+#pragma unroll
+        for (int j = 0; j < L::QPW; ++j) {
+            const int row = cw * 32 + j * L::RPI + ld_rsub;            // 0..127 over the four compute waves
+            const int head = (row >> 4) < hcount ? (row >> 4) : 0;
+            async_load_16B_addr(qb + (size_t)(head * kM + (row & 15)) * L::ROWB + ((ld_pos ^ (row & 15)) * 16),
+                                smem_lds + (cw * 32 + j * L::RPI) * L::ROWB);
+        }
+        wait_vmcnt<0>();
+    }
+    __builtin_amdgcn_s_barrier();                   // K(t_begin) is in LDS
     if (wave_active) {
         qk_tile(t_begin);
         float mloc = -INFINITY;
