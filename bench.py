@@ -348,7 +348,7 @@ def main():
         "kernel_us": {"sdpa_partial": round(sdpa_us, 2), "sdpa_combine": round(comb_us, 2),
                       "gdn_forward_tape": round(fwd_us, 2), "tape_replay_batched_36_layers": round(rep_us, 2)},
         "roofline": {
-            "kernel": "sdpa_partial_pc_kernel<bf16,256>",
+            "kernel": "sdpa_partial_kernel<bf16,256>",
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,

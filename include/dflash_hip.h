@@ -240,7 +240,7 @@ int dflash_sdpa_block_causal_append(void* stream,
  * append entry: read from there, stored into the pages that hold keys len..len+M-1 (which
  * the table must already map), and len_dev counts the rows already cached, block excluded.
  * No additive mask.  Returns DFLASH_NOT_SUPPORTED for a page size the kernel does not
- * take or a sequence so long that one workgroup's span exceeds 512 pages.
+ * take.
  * ---------------------------------------------------------------------- */
 int dflash_sdpa_block_causal_paged(void* stream,
                                    const void* q, void* k_pool, void* v_pool,

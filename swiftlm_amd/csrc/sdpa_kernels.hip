@@ -6,11 +6,11 @@
 //   * all query heads of a GQA group (up to 8 heads x 16 block rows = 128 rows)
 //     share one pass over their KV head's rows, so K/V are read once;
 //   * the key axis is split over enough workgroups to cover every CU (split-KV),
-//     each writing an unnormalised partial (O, max, sum); a second small kernel
-//     combines the splits and emits O and the logsumexp;
-//   * K/V tiles of 64 keys are double-buffered in LDS (prefetch of tile i+1 is in
-//     flight while tile i is multiplied); Q K^T and P V run on bf16/f16 MFMA
-//     (v_mfma_f32_32x32x16) with the online softmax held in registers.
+//     each writing a partial (O / l, max, l); a second small kernel combines the
+//     splits and emits O and the logsumexp;
+//   * K/V tiles of 32 keys go HBM -> LDS directly, several tiles ahead, requested
+//     by two waves that do nothing else; four other waves run Q K^T and P V on
+//     bf16/f16 MFMA (v_mfma_f32_32x32x16) with the online softmax in registers.
 //
 // MFMA operand conventions used below (wave of 64 lanes, c = lane % 32,
 // h = lane / 32):  A (32 x 16) lane holds row c, k-elements 8h..8h+7;
@@ -44,9 +44,8 @@ typedef __attribute__((ext_vector_type(4))) _Float16 f16x4_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;   // one 16-byte global/LDS access
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
 
-constexpr int kSdpaThreads = 256;
+constexpr int kCombineThreads = 256;
 constexpr int kBN = 32;             // keys per tile
-constexpr int kStages = 4;          // LDS tile buffers in flight
 constexpr int kM = 16;              // block rows per head
 constexpr int kHeadsPerWG = 8;      // query heads sharing one K/V pass
 constexpr int kMaxSplits = 512;
@@ -101,24 +100,6 @@ struct SdpaArgs {
     int page_shift, table_stride, num_pages;
 };
 
-constexpr int kPageSlots = 512;     // page-table entries one workgroup keeps in LDS (its own span of the sequence)
-
-// LDS plan of the partial kernel.  A stage holds one tile of kBN keys: the K rows
-// followed by the V rows, both row-major [key][D] exactly as in HBM but with the
-// 16-byte pieces of each row permuted (XOR swizzle) so that the MFMA operand reads
-// below hit every bank once.  kStages stages are in flight.
-template <int D> struct SdpaLds {
-    static constexpr int ROWB = D * 2;               // bytes per K or V row
-    static constexpr int CPR = D / 8;                // 16-byte pieces per row
-    static constexpr int RPI = 64 / CPR;             // rows covered by one wave-wide 1 KB load
-    static constexpr int K_BYTES = kBN * ROWB;
-    static constexpr int STAGE = 2 * K_BYTES;
-    static constexpr int LPW = (kBN / RPI) / 4;      // load instructions per wave per tile and operand
-    static constexpr int EROW = D * 2 + 16;          // epilogue O row pitch, bytes
-    static constexpr int EPI = 4 * 32 * EROW;
-    static constexpr int BYTES = kStages * STAGE > EPI ? kStages * STAGE : EPI;
-};
-
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 typedef __attribute__((address_space(3))) void lds_void_t;
@@ -157,577 +138,62 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt(((N >> 4) << 14) | (0xF << 8) | (0x7 << 4) | (N & 0xF));
 }
 
-// Grid: x = split, y = kv head * groups_per_kv + head group, z = batch.
-//
-// Data movement: K/V rows go HBM -> LDS directly (global_load_lds_dwordx4, no VGPR
-// staging), kStages-1 tiles ahead of the tile being multiplied.  A wave-wide load
-// deposits 64 x 16 B contiguously in LDS in lane order, so the swizzle is applied on
-// the way in: lane l, which fills piece l % CPR of its row, fetches piece
-// (l % CPR) ^ f(row) from HBM.  K uses f = row % 16 (conflict-free ds_read_b128 of
-// one piece per key row across 16 lanes); V uses f = 4 * (row % 4) (conflict-free
-// ds_read_b64_tr_b16 of 4 key rows x 32 B per 16-lane group).
-// V^T operands come from the transposing LDS read: in each 16-lane group, lane
-// 4*j + q supplies the address of 4 channels of key row j; lane i receives channel
-// (i % 4) of the address given by lane 4*r + i/4 as its r-th element, i.e. four
-// consecutive keys of channel d0 + i when lane 4*j + q points at V[k0 + j][d0 + 4q].
-// MASKED adds the reference's optional additive mask: a key is used when it passes the causal rule
-// and its mask value is at least the lowest finite value of the input type, and the mask value is
-// added to the scaled score (DFlashKernels.swift:550-553, :614-623).  The mask is read with plain
-// loads inside the softmax; that instantiation is for signature parity, not for speed.
-template <typename Tag, int D, bool MASKED, bool PAGED>
-__global__ __launch_bounds__(kSdpaThreads, 1) void sdpa_partial_kernel(SdpaArgs A) {
-    typedef typename Tag::vec8 vec8;
-    typedef SdpaLds<D> L;
-    constexpr int KSTEPS = D / 16;     // MFMA k-steps over the head dimension
-    constexpr int DB = D / 32;         // 32-wide output blocks over the head dimension
-
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    // LDS byte address of smem (what M0 and the ds_* instructions use)
-    const uint32_t smem_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int c = lane & 31, h = lane >> 5;
-    const int split = blockIdx.x;
-    const int hk = blockIdx.y / A.groups_per_kv;
-    const int hg0 = (blockIdx.y % A.groups_per_kv) * kHeadsPerWG;   // first head of the group handled here
-    const int b = blockIdx.z;
-    const int hcount = (A.G - hg0) < kHeadsPerWG ? (A.G - hg0) : kHeadsPerWG;
-
-    int Nb = A.kv_len_dev ? A.kv_len_dev[b] + A.len_bias : A.N;
-    Nb = Nb < kM ? kM : (Nb > A.N ? A.N : Nb);
-    const int nt = (Nb + kBN - 1) / kBN;
-    const int t_begin = (int)(((long)split * nt) / A.S);
-    const int t_end = (int)(((long)(split + 1) * nt) / A.S);
-
-    // this wave's query rows: heads 2*wave, 2*wave+1 of the group, 16 rows each
-    const int head_in_group = 2 * wave + (c >> 4);
-    const bool row_valid = head_in_group < hcount;
-    const bool wave_active = 2 * wave < hcount;
-    const int hq = hk * A.G + hg0 + head_in_group;
-    const int qi = c & 15;
-    const size_t row_id = ((size_t)b * A.Hq + hq) * kM + qi;   // valid only when row_valid
-
-    // dense: the head's rows are contiguous; paged: the head's slice of page 0, pages are added per tile
-    const size_t head_off = PAGED ? (size_t)hk * A.kv_head_stride * 2
-                                  : ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
-    const unsigned char* kbase = reinterpret_cast<const unsigned char*>(A.k) + head_off;
-    const unsigned char* vbase = reinterpret_cast<const unsigned char*>(A.v) + head_off;
-    // Paged: byte offset of key n's row from kbase / vbase.  The entries of this workgroup's span are kept
-    // in LDS behind the tile ring (filled below, once the span is known); entries are clamped to the pool.
-    int32_t* ptab = reinterpret_cast<int32_t*>(smem + L::BYTES);
-    const int page_mask = PAGED ? (1 << A.page_shift) - 1 : 0;
-    int page0 = 0;                                      // first page of this workgroup's span
-    auto clamp_page = [&](int e) { return e < 0 ? 0 : (e >= A.num_pages ? A.num_pages - 1 : e); };
-    auto row_off = [&](int key) -> size_t {
-        if constexpr (PAGED)
-            return (size_t)ptab[(key >> A.page_shift) - page0] * (size_t)A.kv_batch_stride * 2 + (size_t)(key & page_mask) * L::ROWB;
-        else
-            return (size_t)key * L::ROWB;
-    };
-
-    // Fused append: keys Nb-16 .. Nb-1 are read from k_new / v_new, and one workgroup per KV head
-    // stores them into the cache rows they stand for.
-    const bool fused = A.k_new != nullptr;
-    const int cache_rows = fused ? Nb - kM : Nb;       // keys below this index are read from the cache
-    const unsigned char* knew = reinterpret_cast<const unsigned char*>(A.k_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
-    const unsigned char* vnew = reinterpret_cast<const unsigned char*>(A.v_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
-    if (fused && A.k_cache && split == 0 && hg0 == 0) {
-        const u32x4_t* ksrc = reinterpret_cast<const u32x4_t*>(knew);
-        const u32x4_t* vsrc = reinterpret_cast<const u32x4_t*>(vnew);
-        if constexpr (PAGED) {
-            // the 16 rows may straddle a page boundary: each row looks its page up (read from the table itself:
-            // this workgroup's LDS span covers the start of the sequence, not its end)
-            for (int i = tid; i < kM * L::CPR; i += kSdpaThreads) {
-                const int key = cache_rows + i / L::CPR;
-                const int page = clamp_page(A.page_table[(size_t)b * A.table_stride + (key >> A.page_shift)]);
-                const size_t off = head_off + (size_t)page * (size_t)A.kv_batch_stride * 2 + (size_t)(key & page_mask) * L::ROWB +
-                                   (size_t)(i % L::CPR) * 16;
-                *reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.k_cache) + off) = ksrc[i];
-                *reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.v_cache) + off) = vsrc[i];
-            }
-        } else {
-            const size_t head = head_off + (size_t)cache_rows * L::ROWB;
-            u32x4_t* kd = reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.k_cache) + head);
-            u32x4_t* vd = reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.v_cache) + head);
-            for (int i = tid; i < kM * L::CPR; i += kSdpaThreads) { kd[i] = ksrc[i]; vd[i] = vsrc[i]; }
-        }
-    }
-
-    if (t_begin >= t_end) {   // empty split: tell the combine kernel to ignore it
-        if (row_valid && h == 0) {
-            A.part_m[row_id * A.S + split] = -INFINITY;
-            A.part_l[row_id * A.S + split] = 0.f;
-        }
-        return;
-    }
-
-    if constexpr (PAGED) {
-        // this workgroup's keys t_begin*kBN .. min(t_end*kBN, Nb) - 1 and the pages they live in
-        page0 = (t_begin * kBN) >> A.page_shift;
-        const int last_key = (t_end * kBN < Nb ? t_end * kBN : Nb) - 1;
-        int npg = (last_key >> A.page_shift) - page0 + 1;                // the host checks that the span fits
-        npg = npg < kPageSlots ? npg : kPageSlots;
-        for (int i = tid; i < npg; i += kSdpaThreads) ptab[i] = clamp_page(A.page_table[(size_t)b * A.table_stride + page0 + i]);
-        __syncthreads();
-    }
-
-    // ---- asynchronous tile loads ------------------------------------------------
-    // Load instruction j of this wave covers rows (4*j + wave) * RPI .. + RPI - 1 of the tile.
-    // The per-lane part of each address (row within the tile, swizzled piece) is fixed, so it is
-    // computed once; a tile that lies entirely inside the sequence only moves the scalar base.
-    const int ld_rsub = lane / L::CPR;           // row within the instruction's row group
-    const int ld_pos = lane % L::CPR;            // 16-byte slot this lane fills
-    uint32_t ld_off_k[L::LPW], ld_off_v[L::LPW];
-#pragma unroll
-    for (int j = 0; j < L::LPW; ++j) {
-        const int row = (4 * j + wave) * L::RPI + ld_rsub;
-        ld_off_k[j] = (uint32_t)row * L::ROWB + (uint32_t)((ld_pos ^ (row & 15)) * 16);
-        ld_off_v[j] = (uint32_t)row * L::ROWB + (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
-    }
-    // Piece j (of LPW) of tile t: one K and one V load instruction of this wave.
-    auto issue_part = [&](int t, int j) {
-        const uint32_t stage_lds = smem_lds + ((t - t_begin) % kStages) * L::STAGE;
-        const int key0 = t * kBN;
-        const int rg = (4 * j + wave) * L::RPI;
-        if (key0 + kBN <= cache_rows) {          // uniform: whole tile comes from the cache
-            const size_t toff = row_off(key0);   // a tile never straddles a page (page sizes are multiples of kBN)
-            const unsigned char* kt = uniform_ptr(kbase + toff);
-            const unsigned char* vt = uniform_ptr(vbase + toff);
-            async_load_16B(kt, ld_off_k[j], stage_lds + rg * L::ROWB);
-            async_load_16B(vt, ld_off_v[j], stage_lds + L::K_BYTES + rg * L::ROWB);
-        } else {
-            // Tail tile: rows past the end re-read the last key (masked later); with a fused append
-            // the block's own 16 rows are taken from k_new / v_new instead of the cache.
-            const int row = rg + ld_rsub;
-            int key = key0 + row;
-            key = key < Nb ? key : Nb - 1;
-            const uint32_t pk = (uint32_t)((ld_pos ^ (row & 15)) * 16);
-            const uint32_t pv = (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
-            const size_t roff = row_off(key < cache_rows ? key : (cache_rows > 0 ? cache_rows - 1 : 0));
-            const unsigned char* ksrc = key < cache_rows ? kbase + roff : knew + (size_t)(key - cache_rows) * L::ROWB;
-            const unsigned char* vsrc = key < cache_rows ? vbase + roff : vnew + (size_t)(key - cache_rows) * L::ROWB;
-            async_load_16B_addr(ksrc + pk, stage_lds + rg * L::ROWB);
-            async_load_16B_addr(vsrc + pv, stage_lds + L::K_BYTES + rg * L::ROWB);
-        }
-    };
-    auto issue_tile = [&](int t) {
-#pragma unroll
-        for (int j = 0; j < L::LPW; ++j) issue_part(t, j);
-    };
-    constexpr int LD_PER_TILE = 2 * L::LPW;      // vmcnt events per tile and wave
-
-    // Tile 0 goes out first, then Q, then tile 1; tile 0 and Q are awaited together (one memory
-    // round trip).  Q takes the same road as the tiles, HBM -> LDS with 1 KB per wave instruction:
-    // fetched straight into the B-operand layout (16 bytes per lane from 32 rows 512 bytes apart) it
-    // costs 2 us of uncoalesced requests per workgroup.  Each wave parks its own 32 rows, swizzled
-    // like a K tile, in the part of the ring that tiles 2 and 3 will use, reads them back as
-    // operands, and only then (after the barrier) is tile 2 requested.
-    static_assert(kStages >= 4, "Q is parked in stages 2 and 3");
-    issue_tile(t_begin);
-    const uint32_t q_park = 2 * L::STAGE + wave * 32 * L::ROWB;
-    if (wave_active) {
-        const int heads_here = (hcount - 2 * wave) >= 2 ? 2 : 1;
-        const unsigned char* qb = reinterpret_cast<const unsigned char*>(A.q) +
-                                  ((size_t)b * A.Hq + hk * A.G + hg0 + 2 * wave) * kM * L::ROWB;
-#pragma unroll
-        for (int j = 0; j < 32 / L::RPI; ++j) {
-            const int row = j * L::RPI + ld_rsub;
-            const int head = (row >> 4) < heads_here ? (row >> 4) : 0;      // an absent head re-reads the first
-            async_load_16B_addr(qb + (size_t)(head * kM + (row & 15)) * L::ROWB + ((ld_pos ^ (row & 15)) * 16),
-                                smem_lds + q_park + j * L::RPI * L::ROWB);
-        }
-    }
-    if (t_begin + 1 < t_end) {
-        issue_tile(t_begin + 1);
-        wait_vmcnt<LD_PER_TILE>();               // tile 0 and Q; tile 1 may still be in flight
-    } else {
-        wait_vmcnt<0>();
-    }
-    asm volatile("" ::: "memory");
-
-    // ---- Q as B operands: column c = query row, k-elements 16*s + 8h .. +7 ----
-    vec8 qreg[KSTEPS];
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s)
-        qreg[s] = *reinterpret_cast<const vec8*>(smem + q_park + c * L::ROWB + (((2 * s + h) ^ (c & 15)) * 16));
-    __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): Q has left LDS before anyone refills stage 2
-    __builtin_amdgcn_s_barrier();                // tile t_begin is in LDS for all waves; Q is in registers
-    if (t_begin + 2 < t_end) issue_tile(t_begin + 2);
-
-    f32x16_t oacc[DB];
-#pragma unroll
-    for (int i = 0; i < DB; ++i)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) oacc[i][v] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
-
-    // per-lane pieces of the operand addresses
-    const int k_rd = c * L::ROWB;                        // K: this lane's key row
-    const int k_sw = c & 15;
-    const int tj = (lane & 15) >> 2, tq = lane & 3;      // V: transposing read, lane = 4*tj + tq in its group
-    const int tg = lane >> 4;                            // group: channel half tg & 1, key half tg >> 1
-    const int v_rd = (4 * (tg >> 1) + tj) * L::ROWB + (tq & 1) * 8;
-    const int v_piece = 2 * (tg & 1) + (tq >> 1);        // 16-byte piece within a 32-channel block
-    const int v_sw = 4 * tj;                             // row % 4 == tj for every row this lane reads
-
-    auto stage_of = [&](int t) -> const unsigned char* { return smem + ((t - t_begin) % kStages) * L::STAGE; };
-    auto load_k = [&](const unsigned char* ks, int s) -> vec8 {
-        return *reinterpret_cast<const vec8*>(ks + k_rd + (((2 * s + h) ^ k_sw) * 16));
-    };
-    // V^T operand of PV step s: output block s % DB, key half s / DB.  The MFMA consumes accumulator
-    // registers 8*ksub .. 8*ksub+7 of S^T, i.e. keys 16*ksub + {4h..4h+3} and 16*ksub + 8 + {4h..4h+3}:
-    // two transposing reads of four keys each.
-    auto load_v = [&](const unsigned char* vs, int s) -> vec8 {
-        const int i = s % DB, ksub = s / DB;
-        const int off = v_rd + ((((4 * i + v_piece)) ^ v_sw) * 16);
-        const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (__attribute__((address_space(3))) s16x4_t*)(vs + off + (16 * ksub) * L::ROWB));
-        const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (__attribute__((address_space(3))) s16x4_t*)(vs + off + (16 * ksub + 8) * L::ROWB));
-        return __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-    };
-    constexpr int kAhead = 4;       // operand reads run this many MFMA steps ahead; sched_barrier pins the order
-
-    // ---- the per-tile work, arranged so that the softmax arithmetic hides behind the MFMAs ----
-    // With one wave per SIMD nothing else fills the VALU while an MFMA runs, and the softmax of a
-    // tile (16 scores per lane: scale, max, 16 quarter-rate exp2, sum, pack) costs about as many
-    // cycles as the tile's 32 MFMAs.  A 32x32x16 MFMA occupies the matrix pipe for 32 cycles after a
-    // 4-cycle issue, and independent VALU instructions of the same wave issue meanwhile.  So each
-    // iteration t runs two blocks:
-    //   phase 1:  S^T(t+1) = K(t+1) Q^T  (MFMA)  with  P(t) = exp2(x(t) - m), row sums, pack  (VALU)
-    //   phase 2:  O^T += V(t)^T P(t)^T   (MFMA)  with  x(t+1) = scale * S^T(t+1), row maximum  (VALU)
-    // where x(t) are tile t's scaled scores.  sched_barrier(0) after every step pins the order.
-    float x[16];                    // scaled (log2 domain) and masked scores of the current tile
-    vec8 pb[2];                     // P^T of the current tile as MFMA operands (two key halves)
-    f32x16_t sacc, sacc1;           // raw scores of the next tile, two accumulation chains
-    float m_pending = -INFINITY;
-
-    // S^T = K Q^T of one tile on its own (first tile only).  Two accumulators: a dependent 32x32x16
-    // MFMA waits out the pipeline latency of its predecessor, two interleaved chains hide half of it.
-    auto qk_tile = [&](int t) {
-        const unsigned char* ks = stage_of(t);
-#pragma unroll
-        for (int v = 0; v < 16; ++v) { sacc[v] = 0.f; sacc1[v] = 0.f; }
-        vec8 ka[KSTEPS];
-#pragma unroll
-        for (int s = 0; s < kAhead; ++s) ka[s] = load_k(ks, s);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s = 0; s < KSTEPS; s += 2) {
-            if (s + kAhead < KSTEPS) { ka[s + kAhead] = load_k(ks, s + kAhead); ka[s + kAhead + 1] = load_k(ks, s + kAhead + 1); }
-            sacc = Tag::mfma(ka[s], qreg[s], sacc);
-            sacc1 = Tag::mfma(ka[s + 1], qreg[s + 1], sacc1);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-
-    // Phase 1 of iteration t.  Tile t_issue (none if negative) is requested meanwhile, a piece at a time.
-    auto exp_qk = [&](int t, auto with_issue, int t_issue) {
-        constexpr bool kIssue = decltype(with_issue)::value;
-        // the requested tile lies entirely inside the cache: only scalar bases move
-        const uint32_t is_lds = smem_lds + ((t_issue - t_begin) % kStages) * L::STAGE;
-        const size_t is_off = kIssue ? row_off(t_issue * kBN) : 0;
-        const unsigned char* is_k = uniform_ptr(kbase + is_off);
-        const unsigned char* is_v = uniform_ptr(vbase + is_off);
-        const unsigned char* ks = stage_of(t + 1);
-        const float m_safe = m_run == -INFINITY ? 0.f : m_run;
-        float psum = 0.f;
-        f32x8_t p0, p1;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) { sacc[v] = 0.f; sacc1[v] = 0.f; }
-        vec8 ka[KSTEPS];
-#pragma unroll
-        for (int s = 0; s < kAhead; ++s) ka[s] = load_k(ks, s);
-        __builtin_amdgcn_sched_barrier(0);
-        constexpr int PAIRS = KSTEPS / 2;           // MFMA pairs in this block
-        constexpr int EPP = 16 / PAIRS;             // scores handled per pair
-        constexpr int IEV = PAIRS / L::LPW;         // a load piece every IEV pairs
-#pragma unroll
-        for (int s = 0; s < KSTEPS; s += 2) {
-            if (s + kAhead < KSTEPS) { ka[s + kAhead] = load_k(ks, s + kAhead); ka[s + kAhead + 1] = load_k(ks, s + kAhead + 1); }
-            sacc = Tag::mfma(ka[s], qreg[s], sacc);
-            sacc1 = Tag::mfma(ka[s + 1], qreg[s + 1], sacc1);
-            const int pr = s / 2;
-#pragma unroll
-            for (int e = pr * EPP; e < (pr + 1) * EPP; ++e) {
-                const float pe = fast_exp2(x[e] - m_safe);
-                psum += pe;
-                if (e < 8) p0[e] = pe; else p1[e - 8] = pe;
-            }
-            if ((pr + 1) * EPP == 8) pb[0] = Tag::pack(p0);
-            if constexpr (kIssue) {
-                if (pr % IEV == 0) {
-                    const int rg = (4 * (pr / IEV) + wave) * L::RPI;
-                    async_load_16B(is_k, ld_off_k[pr / IEV], is_lds + rg * L::ROWB);
-                    async_load_16B(is_v, ld_off_v[pr / IEV], is_lds + L::K_BYTES + rg * L::ROWB);
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        pb[1] = Tag::pack(p1);
-        l_run += psum;
-    };
-
-    // Phase 2 of iteration t: returns the running maximum of x(t+1) over this lane's 16 scores.
-    auto pv_scale = [&](int t) -> float {
-        const unsigned char* vs = stage_of(t) + L::K_BYTES;
-        vec8 va[KSTEPS];
-#pragma unroll
-        for (int s = 0; s < kAhead; ++s) va[s] = load_v(vs, s);
-        __builtin_amdgcn_sched_barrier(0);
-        float mloc = -INFINITY;
-        constexpr int EPS = 16 / KSTEPS;            // scores handled per step
-        constexpr int LAG = 2;                      // steps left to the last score MFMA before its result is read
-#pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) {
-            if (s + kAhead < KSTEPS) va[s + kAhead] = load_v(vs, s + kAhead);
-            oacc[s % DB] = Tag::mfma(va[s], pb[s / DB], oacc[s % DB]);
-            if (s >= LAG) {
-#pragma unroll
-                for (int e = (s - LAG) * EPS; e < (s - LAG + 1) * EPS; ++e) {
-                    x[e] = (sacc[e] + sacc1[e]) * A.scale_log2;
-                    mloc = fmaxf(mloc, x[e]);
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-#pragma unroll
-        for (int e = (KSTEPS - LAG) * EPS; e < 16; ++e) {
-            x[e] = (sacc[e] + sacc1[e]) * A.scale_log2;
-            mloc = fmaxf(mloc, x[e]);
-        }
-        return mloc;
-    };
-
-    // Masks on x (tail tiles: the causal rule; MASKED: the additive mask as well) and the row maximum
-    // over both half-waves.  mloc is the maximum of the unmasked scores.
-    auto mask_and_max = [&](int t, float mloc) -> float {
-        const int key0 = t * kBN;
-        const bool need_mask = (key0 + kBN) > (Nb - kM);
-        if (MASKED || need_mask) {                  // uniform
-            const int last_visible = Nb - kM + qi;  // row qi sees keys 0 .. Nb-16+qi
-            float mk[16];
-            if constexpr (MASKED) {
-                const uint16_t* mrow = A.mask + row_id * (size_t)A.N;
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    int key = key0 + 8 * (v >> 2) + 4 * h + (v & 3);
-                    key = key < A.N ? key : A.N - 1;               // keys past the end fail the causal rule anyway
-                    mk[v] = row_valid ? Tag::to_f32(mrow[key]) : 0.f;
-                }
-            }
-            mloc = -INFINITY;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                if constexpr (MASKED) {
-                    // -inf (or NaN) drops the key; a finite mask value, however low, keeps it in the softmax
-                    x[v] = mk[v] >= -3.4028234663852886e38f ? fmaxf(fmaf(mk[v], 1.4426950408889634f, x[v]), -3.4028234663852886e38f)
-                                                             : -INFINITY;
-                }
-                const int key = key0 + 8 * (v >> 2) + 4 * h + (v & 3);
-                x[v] = key <= last_visible ? x[v] : -INFINITY;
-                mloc = fmaxf(mloc, x[v]);
-            }
-        }
-        return fmaxf(mloc, __shfl_xor(mloc, 32));
-    };
-
-    // Lazy rescale: the exponent reference m_run only moves when a tile's maximum exceeds it by more
-    // than kRescaleLog2 (P then stays below 2^kRescaleLog2, harmless in fp32/bf16).  Rows that are
-    // still empty take the new reference at once; if rows that already accumulated data must move,
-    // false is returned and the caller rescales the accumulators OUTSIDE the hot loop.  (With the
-    // rescale written inside it the register allocator keeps a VGPR copy of all 128 accumulator
-    // registers and refreshes it on every iteration.)
-    auto accept_max = [&](float ml) -> bool {
-        const bool bump = ml > m_run + kRescaleLog2;        // also true for the first finite maximum
-        if (__builtin_amdgcn_ballot_w64(bump && m_run != -INFINITY) != 0) {
-            m_pending = ml;
-            return false;
-        }
-        if (bump) m_run = ml;
-        return true;
-    };
-
-    // P(t) from x(t) without anything to hide behind (last tile)
-    auto exp_tile = [&]() {
-        const float m_safe = m_run == -INFINITY ? 0.f : m_run;
-        float psum = 0.f;
-        f32x8_t p0, p1;
-#pragma unroll
-        for (int v = 0; v < 8; ++v) {
-            p0[v] = fast_exp2(x[v] - m_safe);
-            p1[v] = fast_exp2(x[v + 8] - m_safe);
-            psum += p0[v] + p1[v];
-        }
-        l_run += psum;
-        pb[0] = Tag::pack(p0);
-        pb[1] = Tag::pack(p1);
-    };
-    auto pv_tile = [&](int t) {
-        const unsigned char* vs = stage_of(t) + L::K_BYTES;
-        vec8 va[KSTEPS];
-#pragma unroll
-        for (int s = 0; s < kAhead; ++s) va[s] = load_v(vs, s);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) {
-            if (s + kAhead < KSTEPS) va[s + kAhead] = load_v(vs, s + kAhead);
-            oacc[s % DB] = Tag::mfma(va[s], pb[s / DB], oacc[s % DB]);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-
-    // ---- first tile: scores and their maximum ----
-    if (wave_active) {
-        qk_tile(t_begin);
-        float mloc = -INFINITY;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            x[v] = (sacc[v] + sacc1[v]) * A.scale_log2;
-            mloc = fmaxf(mloc, x[v]);
-        }
-        accept_max(mask_and_max(t_begin, mloc));   // rows are empty: cannot ask for a rescale
-    }
-    int t = t_begin;
-    const int t_last = t_end - 1;
-    while (t < t_last) {
-        bool jumped = false;
-        for (; t < t_last; ++t) {
-            // tile t+1 has landed once at most (tiles issued after it) * LD_PER_TILE loads are outstanding
-            const int later = (t_last - 1 - t) < (kStages - 3) ? (t_last - 1 - t) : (kStages - 3);
-            if (later >= 2) wait_vmcnt<2 * LD_PER_TILE>();
-            else if (later == 1) wait_vmcnt<LD_PER_TILE>();
-            else wait_vmcnt<0>();
-            __builtin_amdgcn_s_barrier();          // tile t+1 is in LDS for everyone; everyone is done with tile t-1
-            const int t_issue = (t + kStages - 1 < t_end) ? t + kStages - 1 : -1;   // refills the stage tile t-1 used
-            const bool spread = t_issue >= 0 && (t_issue + 1) * kBN <= cache_rows;  // requested between the MFMAs
-            if (t_issue >= 0 && !(spread && wave_active)) issue_tile(t_issue);      // tail tile, or a wave without rows
-            if (wave_active) {
-                if (spread) exp_qk(t, std::true_type{}, t_issue);
-                else exp_qk(t, std::false_type{}, 0);
-                const float mloc = pv_scale(t);
-                if (!accept_max(mask_and_max(t + 1, mloc))) {
-                    jumped = true;
-                    break;
-                }
-            }
-        }
-        if (jumped) {                              // cold: move the exponent reference of the rows that jumped
-            const bool bump = m_pending > m_run + kRescaleLog2;
-            const float alpha = (bump && m_run != -INFINITY) ? fast_exp2(m_run - m_pending) : 1.f;
-            if (bump) m_run = m_pending;
-            l_run *= alpha;
-            // The accumulators live in AGPRs inside the loop and this multiply needs them in VGPRs.  Pinning them
-            // to AGPRs on both sides of the multiply makes the compiler copy them HERE; without the pins it
-            // refreshed a VGPR copy of all of them at the end of every loop iteration (128 v_accvgpr_read that
-            // wait for the last MFMA: 0.3 us per tile).
-#pragma unroll
-            for (int i = 0; i < DB; ++i) asm volatile("" : "+a"(oacc[i]));
-#pragma unroll
-            for (int i = 0; i < DB; ++i)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) oacc[i][v] *= alpha;
-#pragma unroll
-            for (int i = 0; i < DB; ++i) asm volatile("" : "+a"(oacc[i]));
-            ++t;                                   // x already holds tile t+1's scores
-        }
-    }
-    if (wave_active) {                             // last tile: nothing left to score
-        exp_tile();
-        pv_tile(t_last);
-    }
-    __syncthreads();          // the tile buffers are free for the epilogue
-
-    // ---- epilogue: partial statistics and O rows (through LDS for coalesced stores) ----
-    const float l_tot = l_run + __shfl_xor(l_run, 32);
-    if (row_valid && h == 0) {
-        A.part_m[row_id * A.S + split] = m_run;
-        A.part_l[row_id * A.S + split] = l_tot;
-    }
-    if (wave_active) {
-        // Partial rows are stored NORMALISED (O / l): the reference keeps them unnormalised in the input type
-        // (DFlashKernels.swift:647) with exponents taken against each block's exact maximum; here the exponent
-        // reference may lag the maximum by 2^kRescaleLog2 and a split spans hundreds of keys, so the raw sums can
-        // pass the largest f16 value.  The combine kernel weights by l accordingly.
-        const float inv_l = l_tot > 0.f ? 1.f / l_tot : 0.f;
-        // Rows are rounded to the input type first and staged as such: lane (c, h) holds 4 consecutive
-        // channels of row c per accumulator quad (8 bytes); the row pitch of D*2 + 16 bytes keeps the
-        // 8-byte writes and the 16-byte reads below spread over the banks.
-        unsigned char* os = smem + wave * 32 * L::EROW;
-#pragma unroll
-        for (int i = 0; i < DB; ++i)
-#pragma unroll
-            for (int v4 = 0; v4 < 4; ++v4) {
-                const f32x4_t o4 = {oacc[i][4 * v4] * inv_l, oacc[i][4 * v4 + 1] * inv_l, oacc[i][4 * v4 + 2] * inv_l,
-                                    oacc[i][4 * v4 + 3] * inv_l};
-                const u32x2_t pk = __builtin_bit_cast(u32x2_t, Tag::pack4(o4));      // hardware round-to-nearest-even
-                *reinterpret_cast<u32x2_t*>(os + c * L::EROW + (32 * i + 8 * v4 + 4 * h) * 2) = pk;
-            }
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): LDS writes of this wave are visible to it
-        const int rows = (hcount - 2 * wave) >= 2 ? 32 : 16;        // this wave's valid rows (whole heads)
-        const size_t rid0 = ((size_t)b * A.Hq + hk * A.G + hg0 + 2 * wave) * kM;   // rows are consecutive
-        constexpr int PER_ROW = D / 8;                              // lanes per row, 8 channels (16 bytes) each
-        constexpr int RPP = 64 / PER_ROW;                           // rows per pass of the wave
-        const int rsub = lane / PER_ROW, d = (lane % PER_ROW) * 8;
-        uint16_t* dst = A.part_o + ((size_t)split * A.rows_total + rid0) * D + d;
-#pragma unroll
-        for (int r0 = 0; r0 < 32; r0 += 8 * RPP) {
-            u32x4_t o[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) o[u] = *reinterpret_cast<const u32x4_t*>(os + (r0 + u * RPP + rsub) * L::EROW + d * 2);
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int r = r0 + u * RPP + rsub;
-                if (r < rows) *reinterpret_cast<u32x4_t*>(dst + (size_t)r * D) = o[u];
-            }
-        }
-    }
-}
-
 // ---------------------------------------------------------------------------
-// Producer/consumer form of the partial kernel (dense and fused-append calls).
+// The partial kernel.  Grid: x = split, y = kv head * groups_per_kv + head group, z = batch.
 //
-// A wave that issues HBM -> LDS loads is held at each load until the memory pipeline takes it; in the
-// streaming steady state that is most of a tile's transfer time, and a wave that is held cannot feed
-// its MFMAs.  Here waves 0..3 only compute and waves 4..5 only request tiles and wait for them, so the
-// holds fall on waves with nothing else to do.  Six waves put two on a SIMD, i.e. 256 registers per
-// wave: Q (64 registers per lane in the kernel above) stays in LDS and is read per k-step like K.
+// Roles.  A wave that issues HBM -> LDS loads is held at each load until the memory pipeline takes it; in the
+// streaming steady state that is most of a tile's transfer time, and a wave that is held cannot feed its
+// MFMAs.  So waves 0..3 only compute (32 query rows each: two heads of the group) and waves 4..5 only request
+// tiles and wait for them: the holds fall on waves with nothing else to do.  Six waves put two on a SIMD, i.e.
+// 256 registers per wave, of which the O^T accumulators take 128 at D = 256; Q therefore stays in LDS and is
+// read per k-step like K.
 //
-// LDS: Q [128 rows] | K ring, kPcSlots tiles | V ring, kPcSlots tiles.  K and V advance separately because
-// the scores run one tile ahead of the PV product: iteration t needs V(t) and K(t+1) ("group t").
-// Producers: request K(t0), group t0, group t0+1 (each compute wave requests its own Q rows meanwhile); then per iteration t: wait for group t, barrier,
-// request group t+2 (V(t+2) into the slot of V(t-1), K(t+3) into the slot of K(t), both free after
-// the barrier).  One barrier per iteration, shared by all six waves.
+// Data movement.  K/V rows go HBM -> LDS directly (global_load_lds_dwordx4, no VGPR staging).  A wave-wide load
+// deposits 64 x 16 B contiguously in LDS in lane order, so the bank swizzle is applied on the way in: lane l,
+// which fills piece l % CPR of its row, fetches piece (l % CPR) ^ f(row) from HBM.  K and Q use f = row % 16
+// (conflict-free ds_read_b128 of one piece per row across 16 lanes); V uses f = 4 * (row % 4) (conflict-free
+// ds_read_b64_tr_b16 of 4 key rows x 32 B per 16-lane group).  V^T operands come from that transposing read:
+// in each 16-lane group, lane 4*j + q supplies the address of 4 channels of key row j; lane i receives channel
+// (i % 4) of the address given by lane 4*r + i/4 as its r-th element, i.e. four consecutive keys of channel
+// d0 + i when lane 4*j + q points at V[k0 + j][d0 + 4q].
+//
+// LDS: Q [128 rows] | K ring, kRingSlots tiles | V ring, kRingSlots tiles.  K and V advance separately because
+// the scores run one tile ahead of the PV product: iteration t needs V(t) and K(t+1) ("group t").  Producers:
+// request K(t0), Q, group t0, group t0+1; then per iteration
+// t: wait for group t, barrier, request group t+2 (V(t+2) into the slot of V(t-1), K(t+3) into the slot of
+// K(t), both free after the barrier).  One barrier per iteration, shared by all six waves.
+//
+// MASKED adds the reference's optional additive mask: a key is used when it passes the causal rule and its mask
+// value is at least the lowest finite value of the input type, and the mask value is added to the scaled score
+// (DFlashKernels.swift:550-553, :614-623).  The mask is read with plain loads inside the softmax; that
+// instantiation is for signature parity, not for speed.  PAGED reads K/V through a page table.
 // ---------------------------------------------------------------------------
-constexpr int kPcThreads = 384;
-constexpr int kPcSlots = 3;
+constexpr int kPartialThreads = 384;    // 4 compute waves + 2 producer waves
+constexpr int kRingSlots = 3;           // tiles per ring
 
-template <int D> struct PcLds {
+template <int D> struct SdpaLds {
     static constexpr int ROWB = D * 2;
     static constexpr int CPR = D / 8;
     static constexpr int RPI = 64 / CPR;                     // rows per 1 KB load instruction
     static constexpr int KT = kBN * ROWB;                    // bytes of one K (or V) tile
     static constexpr int Q_BYTES = 4 * 32 * ROWB;            // 32 query rows per compute wave
     static constexpr int K_RING = Q_BYTES;
-    static constexpr int V_RING = Q_BYTES + kPcSlots * KT;
+    static constexpr int V_RING = Q_BYTES + kRingSlots * KT;
     static constexpr int LPP = (kBN / RPI) / 2;              // load instructions per producer wave per K (or V) tile
-    static constexpr int QPW = 32 / RPI;                     // load instructions per compute wave for its Q rows
-    static constexpr int EROW = D * 2 + 16;
+    static constexpr int QPP = (128 / RPI) / 2;              // ... for Q
+    static constexpr int EROW = D * 2 + 16;                  // epilogue O row pitch, bytes
     static constexpr int EPI = 4 * 32 * EROW;
-    static constexpr int RING_END = Q_BYTES + 2 * kPcSlots * KT;
+    static constexpr int RING_END = Q_BYTES + 2 * kRingSlots * KT;
     static constexpr int BYTES = RING_END > EPI ? RING_END : EPI;
 };
 
-template <typename Tag, int D>
-__global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs A) {
+template <typename Tag, int D, bool MASKED, bool PAGED>
+__global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaArgs A) {
     typedef typename Tag::vec8 vec8;
-    typedef PcLds<D> L;
+    typedef SdpaLds<D> L;
     constexpr int KSTEPS = D / 16;
     constexpr int DB = D / 32;
-    static_assert(4 * L::LPP <= 63 && L::QPW <= 63, "vmcnt is a 6-bit counter");
+    static_assert(4 * L::LPP <= 63, "vmcnt is a 6-bit counter");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t smem_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
@@ -763,20 +229,37 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
     const int qi = c & 15;
     const size_t row_id = ((size_t)b * A.Hq + hq) * kM + qi;
 
-    const size_t head_off = ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
+    // dense: the head's rows are contiguous; paged: the head's slice of page 0, the page is added per tile
+    const size_t head_off = PAGED ? (size_t)hk * A.kv_head_stride * 2
+                                  : ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
     const unsigned char* kbase = reinterpret_cast<const unsigned char*>(A.k) + head_off;
     const unsigned char* vbase = reinterpret_cast<const unsigned char*>(A.v) + head_off;
+    // Byte offset of key n's row from kbase / vbase (the K and V pools share one layout).  Paged: the page comes
+    // from the table, clamped to the pool; a tile never straddles a page (page sizes are multiples of kBN).
+    const int page_mask = PAGED ? (1 << A.page_shift) - 1 : 0;
+    auto row_off = [&](int key) -> size_t {
+        if constexpr (PAGED) {
+            int e = A.page_table[(size_t)b * A.table_stride + (key >> A.page_shift)];
+            e = e < 0 ? 0 : (e >= A.num_pages ? A.num_pages - 1 : e);
+            return (size_t)e * (size_t)A.kv_batch_stride * 2 + (size_t)(key & page_mask) * L::ROWB;
+        } else {
+            return (size_t)key * L::ROWB;
+        }
+    };
+    // Fused append: keys Nb-16 .. Nb-1 are read from k_new / v_new, and one workgroup per KV head stores them
+    // into the cache rows they stand for (paged: the 16 rows may straddle a page, so every row looks its page up).
     const bool fused = A.k_new != nullptr;
-    const int cache_rows = fused ? Nb - kM : Nb;
+    const int cache_rows = fused ? Nb - kM : Nb;       // keys below this index are read from the cache
     const unsigned char* knew = reinterpret_cast<const unsigned char*>(A.k_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
     const unsigned char* vnew = reinterpret_cast<const unsigned char*>(A.v_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
     if (fused && A.k_cache && split == 0 && hg0 == 0) {
-        const size_t head = head_off + (size_t)cache_rows * L::ROWB;
-        u32x4_t* kd = reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.k_cache) + head);
-        u32x4_t* vd = reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.v_cache) + head);
         const u32x4_t* ksrc = reinterpret_cast<const u32x4_t*>(knew);
         const u32x4_t* vsrc = reinterpret_cast<const u32x4_t*>(vnew);
-        for (int i = tid; i < kM * L::CPR; i += kPcThreads) { kd[i] = ksrc[i]; vd[i] = vsrc[i]; }
+        for (int i = tid; i < kM * L::CPR; i += kPartialThreads) {
+            const size_t off = head_off + row_off(cache_rows + i / L::CPR) + (size_t)(i % L::CPR) * 16;
+            *reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.k_cache) + off) = ksrc[i];
+            *reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.v_cache) + off) = vsrc[i];
+        }
     }
 
     if (t_begin >= t_end) {   // empty split: tell the combine kernel to ignore it
@@ -792,10 +275,10 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
         const int pw = wave - 4;
         const int ld_rsub = lane / L::CPR, ld_pos = lane % L::CPR;
         // instruction j of this producer covers rows (2*j + pw) * RPI .. + RPI - 1 of a tile (or of Q)
-        auto issue_rows = [&](const unsigned char* base, bool k_swizzle, int t, uint32_t lds_tile, bool is_k) {
+        auto issue_rows = [&](const unsigned char* base, bool k_swizzle, int t, size_t toff, uint32_t lds_tile, bool is_k) {
             const int key0 = key_of(t);
             if (key0 + kBN <= cache_rows) {              // uniform: whole tile comes from the cache
-                const unsigned char* tp = uniform_ptr(base + (size_t)key0 * L::ROWB);
+                const unsigned char* tp = uniform_ptr(base + toff);
 #pragma unroll
                 for (int j = 0; j < L::LPP; ++j) {
                     const int rg = (2 * j + pw) * L::RPI;
@@ -814,23 +297,46 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
                     key = key < Nb ? key : Nb - 1;
                     const uint32_t sw = k_swizzle ? (uint32_t)((ld_pos ^ (row & 15)) * 16) : (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
                     const unsigned char* nw = is_k ? knew : vnew;
-                    const unsigned char* src = key < cache_rows ? base + (size_t)key * L::ROWB : nw + (size_t)(key - cache_rows) * L::ROWB;
+                    const unsigned char* src = key < cache_rows ? base + row_off(key) : nw + (size_t)(key - cache_rows) * L::ROWB;
                     async_load_16B_addr(src + sw, lds_tile + rg * L::ROWB);
                 }
             }
         };
-        auto issue_k = [&](int t) {
-            if (t < t_end) issue_rows(kbase, true, t, smem_lds + L::K_RING + ((t - t_begin) % kPcSlots) * L::KT, true);
+        auto issue_k = [&](int t, size_t toff) {
+            if (t < t_end) issue_rows(kbase, true, t, toff, smem_lds + L::K_RING + ((t - t_begin) % kRingSlots) * L::KT, true);
         };
-        auto issue_v = [&](int t) {
-            if (t < t_end) issue_rows(vbase, false, t, smem_lds + L::V_RING + ((t - t_begin) % kPcSlots) * L::KT, false);
+        auto issue_v = [&](int t, size_t toff) {
+            if (t < t_end) issue_rows(vbase, false, t, toff, smem_lds + L::V_RING + ((t - t_begin) % kRingSlots) * L::KT, false);
         };
+        // Offset of tile t's first row (a wave-uniform value; paged: one scalar read of the page table).  Inside the
+        // loop it is looked up an iteration before it is used, so the table read never delays a request.
+        auto tile_off = [&](int t) -> size_t { return t < t_end ? row_off(key_of(t)) : 0; };
         // loads of group t still outstanding when one waits for the group before it
         auto group_loads = [&](int t) { return (t < t_end ? L::LPP : 0) + (t + 1 < t_end ? L::LPP : 0); };
 
-        issue_k(t_begin);
-        issue_v(t_begin); issue_k(t_begin + 1);            // group t_begin
-        issue_v(t_begin + 1); issue_k(t_begin + 2);        // group t_begin + 1
+        {
+            const size_t o0 = tile_off(t_begin), o1 = tile_off(t_begin + 1);
+            issue_k(t_begin, o0);
+            // Q: 32 rows per compute wave (heads 2w, 2w+1 of the group), swizzled like a K tile, at w * 32 rows of the
+            // Q area; an absent head re-reads the group's first head (its rows are never stored).  Requested right
+            // behind the first K tile: the first scores need both, and nothing else should queue ahead of them.
+            // (Requested by the compute waves instead, Q lands behind the producers' whole opening burst.)
+            {
+                const unsigned char* qb = reinterpret_cast<const unsigned char*>(A.q) + ((size_t)b * A.Hq + hk * A.G + hg0) * kM * L::ROWB;
+#pragma unroll
+                for (int j = 0; j < L::QPP; ++j) {
+                    const int row = (2 * j + pw) * L::RPI + ld_rsub;           // 0..127 over the four compute waves
+                    const int head = (row >> 4) < hcount ? (row >> 4) : 0;
+                    async_load_16B_addr(qb + (size_t)(head * kM + (row & 15)) * L::ROWB + ((ld_pos ^ (row & 15)) * 16),
+                                        smem_lds + (2 * j + pw) * L::RPI * L::ROWB);
+                }
+            }
+            issue_v(t_begin, o0); issue_k(t_begin + 1, o1);     // group t_begin
+            issue_v(t_begin + 1, o1);                           // group t_begin + 1 ...
+        }
+        size_t off_v = tile_off(t_begin + 2);                   // tile whose V the next iteration requests
+        issue_k(t_begin + 2, off_v);                            // ... and its K
+        size_t off_k = tile_off(t_begin + 3);                   // tile whose K the next iteration requests
         {
             const int later = group_loads(t_begin) + group_loads(t_begin + 1);     // 0 .. 4 * LPP
             if (later >= 4 * L::LPP) wait_vmcnt<4 * L::LPP>();
@@ -839,30 +345,32 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
             else if (later >= L::LPP) wait_vmcnt<L::LPP>();
             else wait_vmcnt<0>();
         }
-        __builtin_amdgcn_s_barrier();                       // K(t_begin) is in LDS (and each compute wave's Q rows)
+        __builtin_amdgcn_s_barrier();                       // Q and K(t_begin) are in LDS
         for (int t = t_begin; t <= t_last; ++t) {
             const int later = group_loads(t + 1);
             if (later >= 2 * L::LPP) wait_vmcnt<2 * L::LPP>();
             else if (later >= L::LPP) wait_vmcnt<L::LPP>();
             else wait_vmcnt<0>();
             __builtin_amdgcn_s_barrier();                   // group t is in LDS; iteration t-1 is over for every wave
-            issue_v(t + 2); issue_k(t + 3);                 // group t + 2, into the slots iteration t-1 released
+            issue_v(t + 2, off_v); issue_k(t + 3, off_k);   // group t + 2, into the slots iteration t-1 released
+            off_v = off_k;
+            off_k = tile_off(t + 4);
         }
         return;
     }
 
     // =========================== compute waves ===========================
-    const int k_rd = c * L::ROWB;
+    // per-lane pieces of the operand addresses
+    const int k_rd = c * L::ROWB;                        // K, Q: this lane's row
     const int k_sw = c & 15;
-    const int tj = (lane & 15) >> 2, tq = lane & 3;
-    const int tg = lane >> 4;
+    const int tj = (lane & 15) >> 2, tq = lane & 3;      // V: transposing read, lane = 4*tj + tq in its group
+    const int tg = lane >> 4;                            // group: channel half tg & 1, key half tg >> 1
     const int v_rd = (4 * (tg >> 1) + tj) * L::ROWB + (tq & 1) * 8;
-    const int v_piece = 2 * (tg & 1) + (tq >> 1);
-    const int v_sw = 4 * tj;
+    const int v_piece = 2 * (tg & 1) + (tq >> 1);        // 16-byte piece within a 32-channel block
     const unsigned char* q_rows = smem + cw * 32 * L::ROWB;
 
-    auto k_slot = [&](int t) -> const unsigned char* { return smem + L::K_RING + ((t - t_begin) % kPcSlots) * L::KT; };
-    auto v_slot = [&](int t) -> const unsigned char* { return smem + L::V_RING + ((t - t_begin) % kPcSlots) * L::KT; };
+    auto k_slot = [&](int t) -> const unsigned char* { return smem + L::K_RING + ((t - t_begin) % kRingSlots) * L::KT; };
+    auto v_slot = [&](int t) -> const unsigned char* { return smem + L::V_RING + ((t - t_begin) % kRingSlots) * L::KT; };
     // Operand offsets inside a tile.  The XOR swizzles only touch the low bits of the piece index, so a handful of
     // per-lane offsets plus compile-time constants (folded into the ds_read offset field) cover every k-step:
     //   K, Q: piece (2s+h) ^ (c & 15) = 16 * (s >> 3) + ((2 * (s & 7) + h) ^ (c & 15))
@@ -872,13 +380,15 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
     for (int j = 0; j < 8; ++j) koff[j] = (uint32_t)(k_rd + (((2 * j + h) ^ k_sw) & (L::CPR - 1)) * 16);
 #pragma unroll
     for (int m = 0; m < 4; ++m) voff[m] = (uint32_t)(v_rd + v_piece * 16 + ((m ^ tj) * 64));
-    (void)v_sw;
     auto load_k = [&](const unsigned char* ks, int s) -> vec8 {
         return *reinterpret_cast<const vec8*>(ks + koff[s & 7] + 256 * (s >> 3));
     };
     auto load_q = [&](int s) -> vec8 {
         return *reinterpret_cast<const vec8*>(q_rows + koff[s & 7] + 256 * (s >> 3));
     };
+    // V^T operand of PV step s: output block s % DB, key half s / DB.  The MFMA consumes accumulator registers
+    // 8*ksub .. 8*ksub+7 of S^T, i.e. keys 16*ksub + {4h..4h+3} and 16*ksub + 8 + {4h..4h+3}: two transposing
+    // reads of four keys each.
     auto load_v = [&](const unsigned char* vs, int s) -> vec8 {
         const int i = s % DB, ksub = s / DB;
         const unsigned char* p = vs + voff[i & 3] + 256 * (i >> 2);
@@ -897,11 +407,22 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
 #pragma unroll
         for (int v = 0; v < 16; ++v) oacc[i][v] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
-    float x[16];
-    vec8 pb[2];
-    f32x16_t sacc, sacc1;
+
+    // ---- the per-tile work, arranged so that the softmax arithmetic hides behind the MFMAs ----
+    // With one compute wave per SIMD nothing else fills the VALU while an MFMA runs, and the softmax of a tile
+    // (16 scores per lane: scale, max, 16 quarter-rate exp2, sum, pack) costs about as many cycles as the tile's
+    // 32 MFMAs.  A 32x32x16 MFMA occupies the matrix pipe for 32 cycles after a 4-cycle issue, and independent
+    // VALU instructions of the same wave issue meanwhile.  So each iteration t runs two blocks:
+    //   phase 1:  S^T(t+1) = K(t+1) Q^T  (MFMA)  with  P(t) = exp2(x(t) - m), row sums, pack  (VALU)
+    //   phase 2:  O^T += V(t)^T P(t)^T   (MFMA)  with  x(t+1) = scale * S^T(t+1), row maximum  (VALU)
+    // where x(t) are tile t's scaled scores.  sched_barrier(0) after every step pins the order.
+    float x[16];                    // scaled (log2 domain) and masked scores of the current tile
+    vec8 pb[2];                     // P^T of the current tile as MFMA operands (two key halves)
+    f32x16_t sacc, sacc1;           // raw scores of the next tile, two accumulation chains
     float m_pending = -INFINITY;
 
+    // S^T = K Q^T of one tile on its own (first tile only).  Two accumulators: a dependent 32x32x16 MFMA waits
+    // out the pipeline latency of its predecessor, two interleaved chains hide half of it.
     auto qk_tile = [&](int t) {
         const unsigned char* ks = k_slot(t);
 #pragma unroll
@@ -921,6 +442,7 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
             __builtin_amdgcn_sched_barrier(0);
         }
     };
+    // Phase 1 of iteration t.
     auto exp_qk = [&](int t) {
         const unsigned char* ks = k_slot(t + 1);
         const float m_safe = m_run == -INFINITY ? 0.f : m_run;
@@ -955,6 +477,7 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
         pb[1] = Tag::pack(p1);
         l_run += psum;
     };
+    // Phase 2 of iteration t: returns the running maximum of x(t+1) over this lane's 16 scores.
     auto pv_scale = [&](int t) -> float {
         const unsigned char* vs = v_slot(t);
         vec8 va[KSTEPS];
@@ -984,13 +507,31 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
         }
         return mloc;
     };
+    // Masks on x (tiles that reach the block's own keys: the causal rule; MASKED: the additive mask as well) and
+    // the row maximum over both half-waves.  mloc is the maximum of the unmasked scores.
     auto mask_and_max = [&](int t, float mloc) -> float {
         const int key0 = key_of(t);
-        if ((key0 + kBN) > (Nb - kM)) {            // uniform: the tile reaches into the block's own keys
-            const int last_visible = Nb - kM + qi;
+        const bool need_mask = (key0 + kBN) > (Nb - kM);
+        if (MASKED || need_mask) {                  // uniform
+            const int last_visible = Nb - kM + qi;  // row qi sees keys 0 .. Nb-16+qi
+            float mk[16];
+            if constexpr (MASKED) {
+                const uint16_t* mrow = A.mask + row_id * (size_t)A.N;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    int key = key0 + 8 * (v >> 2) + 4 * h + (v & 3);
+                    key = key < A.N ? key : A.N - 1;               // keys past the end fail the causal rule anyway
+                    mk[v] = row_valid ? Tag::to_f32(mrow[key]) : 0.f;
+                }
+            }
             mloc = -INFINITY;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
+                if constexpr (MASKED) {
+                    // -inf (or NaN) drops the key; a finite mask value, however low, keeps it in the softmax
+                    x[v] = mk[v] >= -3.4028234663852886e38f ? fmaxf(fmaf(mk[v], 1.4426950408889634f, x[v]), -3.4028234663852886e38f)
+                                                             : -INFINITY;
+                }
                 const int key = key0 + 8 * (v >> 2) + 4 * h + (v & 3);
                 x[v] = key <= last_visible ? x[v] : -INFINITY;
                 mloc = fmaxf(mloc, x[v]);
@@ -998,8 +539,13 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
         }
         return fmaxf(mloc, __shfl_xor(mloc, 32));
     };
+    // Lazy rescale: the exponent reference m_run only moves when a tile's maximum exceeds it by more than
+    // kRescaleLog2 (P then stays below 2^kRescaleLog2, harmless in fp32/bf16).  Rows that are still empty take the
+    // new reference at once; if rows that already accumulated data must move, false is returned and the caller
+    // rescales the accumulators OUTSIDE the hot loop.  (With the rescale written inside it the register allocator
+    // keeps a second copy of all 128 accumulator registers and refreshes it on every iteration.)
     auto accept_max = [&](float ml) -> bool {
-        const bool bump = ml > m_run + kRescaleLog2;
+        const bool bump = ml > m_run + kRescaleLog2;        // also true for the first finite maximum
         if (__builtin_amdgcn_ballot_w64(bump && m_run != -INFINITY) != 0) {
             m_pending = ml;
             return false;
@@ -1007,6 +553,7 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
         if (bump) m_run = ml;
         return true;
     };
+    // P(t) from x(t) without anything to hide behind (last tile)
     auto exp_tile = [&]() {
         const float m_safe = m_run == -INFINITY ? 0.f : m_run;
         float psum = 0.f;
@@ -1035,23 +582,7 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
         }
     };
 
-    // Q: this wave's own 32 rows (heads 2w, 2w+1 of the group), swizzled like a K tile, at w * 32 rows of the Q
-    // area.  Each compute wave requests its own rows while the producers are already requesting K and V; nobody
-    // else reads them, so the wave's own wait is all the synchronisation they need.  An absent head re-reads the
-    // group's first head (its rows are never stored).
-    if (wave_active) {
-        const int ld_rsub = lane / L::CPR, ld_pos = lane % L::CPR;
-        const unsigned char* qb = reinterpret_cast<const unsigned char*>(A.q) + ((size_t)b * A.Hq + hk * A.G + hg0) * kM * L::ROWB;
-#pragma unroll
-        for (int j = 0; j < L::QPW; ++j) {
-            const int row = cw * 32 + j * L::RPI + ld_rsub;            // 0..127 over the four compute waves
-            const int head = (row >> 4) < hcount ? (row >> 4) : 0;
-            async_load_16B_addr(qb + (size_t)(head * kM + (row & 15)) * L::ROWB + ((ld_pos ^ (row & 15)) * 16),
-                                smem_lds + (cw * 32 + j * L::RPI) * L::ROWB);
-        }
-        wait_vmcnt<0>();
-    }
-    __builtin_amdgcn_s_barrier();                   // K(t_begin) is in LDS
+    __builtin_amdgcn_s_barrier();                   // Q and K(t_begin) are in LDS
     if (wave_active) {
         qk_tile(t_begin);
         float mloc = -INFINITY;
@@ -1100,7 +631,7 @@ __global__ __launch_bounds__(kPcThreads, 1) void sdpa_partial_pc_kernel(SdpaArgs
     // (the producers' last wait was vmcnt(0)).
     static_assert(L::EPI <= L::V_RING, "the epilogue staging must stay clear of the V ring");
 
-    // ---- epilogue: partial statistics and O rows (as in the kernel above) ----
+    // ---- epilogue: partial statistics and O rows (through LDS for coalesced stores) ----
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     if (row_valid && h == 0) {
         A.part_m[row_id * A.S + split] = m_run;
@@ -1151,12 +682,12 @@ struct CombineArgs {
 };
 
 template <typename Tag, int D>
-__global__ __launch_bounds__(kSdpaThreads) void sdpa_combine_kernel(CombineArgs A) {
+__global__ __launch_bounds__(kCombineThreads) void sdpa_combine_kernel(CombineArgs A) {
     constexpr int TPG = D / 8;                     // threads spanning one row, 8 elements (16 B) each
-    constexpr int NG = kSdpaThreads / TPG;         // split groups walking the partials in parallel
+    constexpr int NG = kCombineThreads / TPG;         // split groups walking the partials in parallel
     constexpr int UNROLL = 4;
     __shared__ float w_s[kMaxSplits];
-    __shared__ float red_s[kSdpaThreads / 64];
+    __shared__ float red_s[kCombineThreads / 64];
     __shared__ float acc_s[NG][D];
 
     const size_t row = blockIdx.x;
@@ -1166,7 +697,7 @@ __global__ __launch_bounds__(kSdpaThreads) void sdpa_combine_kernel(CombineArgs 
 
     // global max
     float mx = -INFINITY;
-    for (int s = tid; s < A.S; s += kSdpaThreads) mx = fmaxf(mx, pm[s]);
+    for (int s = tid; s < A.S; s += kCombineThreads) mx = fmaxf(mx, pm[s]);
     for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
     if ((tid & 63) == 0) red_s[tid >> 6] = mx;
     __syncthreads();
@@ -1174,7 +705,7 @@ __global__ __launch_bounds__(kSdpaThreads) void sdpa_combine_kernel(CombineArgs 
     __syncthreads();
     // weights and denominator
     float lsum = 0.f;
-    for (int s = tid; s < A.S; s += kSdpaThreads) {
+    for (int s = tid; s < A.S; s += kCombineThreads) {
         const float m = pm[s];
         const float w = m == -INFINITY ? 0.f : fast_exp2(m - mx) * pl[s];   // the partial rows are O / l: weight by l
         w_s[s] = w;
@@ -1212,7 +743,7 @@ __global__ __launch_bounds__(kSdpaThreads) void sdpa_combine_kernel(CombineArgs 
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc_s[grp][d8 + e] = acc[e];
     __syncthreads();
-    for (int d = tid; d < D; d += kSdpaThreads) {
+    for (int d = tid; d < D; d += kCombineThreads) {
         float r = 0.f;
 #pragma unroll
         for (int gI = 0; gI < NG; ++gI) r += acc_s[gI][d];
@@ -1256,54 +787,23 @@ static size_t ws_layout(int B, int Hq, int S, int D, size_t* off_m, size_t* off_
     return (o + 255) & ~(size_t)255;
 }
 
-// DFLASH_SDPA_PRODUCERS=0 selects the single-role kernel for every call (A/B runs, and the tests that compare
-// the paged entry, which always uses that kernel, byte for byte with the dense one).  Read at each call.
-static bool use_producer_kernel() {
-    const char* e = getenv("DFLASH_SDPA_PRODUCERS");
-    return !(e && e[0] == '0');
-}
-
-template <typename Tag, int D>
-static int launch_sdpa_pc(hipStream_t st, const SdpaArgs& A, const CombineArgs& C, int B) {
-    typedef PcLds<D> L;
+template <typename Tag, int D, bool MASKED, bool PAGED>
+static int launch_sdpa(hipStream_t st, const SdpaArgs& A, const CombineArgs& C, int B) {
+    typedef SdpaLds<D> L;
     static_assert(L::BYTES <= 160 * 1024, "Q and the tile rings must fit the 160 KB LDS of a gfx950 CU");
-    auto kern = sdpa_partial_pc_kernel<Tag, D>;
+    auto kern = sdpa_partial_kernel<Tag, D, MASKED, PAGED>;
     static const hipError_t attr_rc =
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::BYTES);
     DFLASH_HIP_TRY(attr_rc);
     dim3 grid(A.S, A.Hk * A.groups_per_kv, B);
     {
         LaunchBracket br(DFLASH_KERNEL_SDPA_PARTIAL, st);
-        br.launch(kern, grid, dim3(kPcThreads), L::BYTES, A);
+        br.launch(kern, grid, dim3(kPartialThreads), L::BYTES, A);
     }
     DFLASH_HIP_TRY(hipGetLastError());
     {
         LaunchBracket br(DFLASH_KERNEL_SDPA_COMBINE, st);
-        br.launch(sdpa_combine_kernel<Tag, D>, dim3(B * A.Hq * kM), dim3(kSdpaThreads), 0, C);
-    }
-    DFLASH_HIP_TRY(hipGetLastError());
-    return DFLASH_OK;
-}
-
-template <typename Tag, int D, bool MASKED, bool PAGED>
-static int launch_sdpa(hipStream_t st, const SdpaArgs& A, const CombineArgs& C, int B) {
-    typedef SdpaLds<D> L;
-    constexpr int kLdsBytes = L::BYTES + (PAGED ? kPageSlots * (int)sizeof(int32_t) : 0);
-    static_assert(kLdsBytes <= 160 * 1024, "tile buffers must fit the 160 KB LDS of a gfx950 CU");
-    auto kern = sdpa_partial_kernel<Tag, D, MASKED, PAGED>;
-    // Raise the dynamic LDS limit above the 64 KB default, once per process.
-    static const hipError_t attr_rc =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-    DFLASH_HIP_TRY(attr_rc);
-    dim3 grid(A.S, A.Hk * A.groups_per_kv, B);
-    {
-        LaunchBracket br(DFLASH_KERNEL_SDPA_PARTIAL, st);
-        br.launch(kern, grid, dim3(kSdpaThreads), kLdsBytes, A);
-    }
-    DFLASH_HIP_TRY(hipGetLastError());
-    {
-        LaunchBracket br(DFLASH_KERNEL_SDPA_COMBINE, st);
-        br.launch(sdpa_combine_kernel<Tag, D>, dim3(B * A.Hq * kM), dim3(kSdpaThreads), 0, C);
+        br.launch(sdpa_combine_kernel<Tag, D>, dim3(B * A.Hq * kM), dim3(kCombineThreads), 0, C);
     }
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
@@ -1367,12 +867,6 @@ static int sdpa_common(void* stream, const void* q, const void* k, const void* v
     const int G = Hq / Hk;
     const int groups = (G + kHeadsPerWG - 1) / kHeadsPerWG;
     const int S = choose_splits(B, Hk, groups, N);
-    if (paged) {
-        const int nt = (N + kBN - 1) / kBN;
-        const int span_pages = ((((nt + S - 1) / S) * kBN) >> page_shift) + 2;      // pages one workgroup's keys can touch
-        DFLASH_SUPPORTED(span_pages <= kPageSlots, "sdpa (paged): %d pages per workgroup exceed the %d the kernel keeps", span_pages,
-                         kPageSlots);
-    }
     size_t om, ol;
     const size_t need = ws_layout(B, Hq, S, D, &om, &ol);
     DFLASH_REQUIRE(workspace && workspace_bytes >= need, "sdpa: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
@@ -1400,20 +894,18 @@ static int sdpa_common(void* stream, const void* q, const void* k, const void* v
     C.out = (uint16_t*)out; C.lse = lse; C.S = S;
 
     hipStream_t st = (hipStream_t)stream;
-    if (mask) {
-        if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa<Bf16Tag, 256, true, false>(st, A, C, B) : launch_sdpa<Bf16Tag, 128, true, false>(st, A, C, B);
-        return D == 256 ? launch_sdpa<F16Tag, 256, true, false>(st, A, C, B) : launch_sdpa<F16Tag, 128, true, false>(st, A, C, B);
-    }
-    if (paged) {
-        if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa<Bf16Tag, 256, false, true>(st, A, C, B) : launch_sdpa<Bf16Tag, 128, false, true>(st, A, C, B);
-        return D == 256 ? launch_sdpa<F16Tag, 256, false, true>(st, A, C, B) : launch_sdpa<F16Tag, 128, false, true>(st, A, C, B);
-    }
-    if (use_producer_kernel()) {
-        if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa_pc<Bf16Tag, 256>(st, A, C, B) : launch_sdpa_pc<Bf16Tag, 128>(st, A, C, B);
-        return D == 256 ? launch_sdpa_pc<F16Tag, 256>(st, A, C, B) : launch_sdpa_pc<F16Tag, 128>(st, A, C, B);
-    }
-    if (dtype == DFLASH_BF16) return D == 256 ? launch_sdpa<Bf16Tag, 256, false, false>(st, A, C, B) : launch_sdpa<Bf16Tag, 128, false, false>(st, A, C, B);
-    return D == 256 ? launch_sdpa<F16Tag, 256, false, false>(st, A, C, B) : launch_sdpa<F16Tag, 128, false, false>(st, A, C, B);
+#define DFLASH_SDPA_CASE(MASKED, PAGED)                                                                              \
+    do {                                                                                                             \
+        if (dtype == DFLASH_BF16)                                                                                    \
+            return D == 256 ? launch_sdpa<Bf16Tag, 256, MASKED, PAGED>(st, A, C, B)                               \
+                            : launch_sdpa<Bf16Tag, 128, MASKED, PAGED>(st, A, C, B);                              \
+        return D == 256 ? launch_sdpa<F16Tag, 256, MASKED, PAGED>(st, A, C, B)                                    \
+                        : launch_sdpa<F16Tag, 128, MASKED, PAGED>(st, A, C, B);                                   \
+    } while (0)
+    if (mask) DFLASH_SDPA_CASE(true, false);
+    if (paged) DFLASH_SDPA_CASE(false, true);
+    DFLASH_SDPA_CASE(false, false);
+#undef DFLASH_SDPA_CASE
 }
 
 extern "C" int dflash_sdpa_block_causal(void* stream, const void* q, const void* k, const void* v, void* out,

@@ -351,14 +351,12 @@ def test_verify_stack_steps_match_oracle_and_fused_accept(gpu_lib):
             np.testing.assert_allclose(host(la["out"]), ow, rtol=2e-2, atol=2e-2)
 
 
-def test_verify_stack_paged_equals_dense(gpu_lib, monkeypatch):
+def test_verify_stack_paged_equals_dense(gpu_lib):
     """The verify-step driver with paged K/V pools gives the bytes of the dense driver, step after step,
     and the appended rows sit in the pages the table names."""
     import torch
     from swiftlm_amd.verify_step import HybridVerifyStack, StackConfig
 
-    # the paged entry runs on the single-role attention kernel: pin the dense stack to it for a byte-for-byte comparison
-    monkeypatch.setenv("DFLASH_SDPA_PRODUCERS", "0")
     kw = dict(n_layers=8, attn_every=4, block=16, Hk=2, Hv=4, Dk=128, Dv=32, Hq=4, Hkv=2, D=128, context=150, max_steps=6)
     dense = HybridVerifyStack(StackConfig(**kw), seed=3)
     paged = HybridVerifyStack(StackConfig(page_size=32, **kw), seed=3)

@@ -7,9 +7,7 @@ gathered cache (bf16/f16 outputs within 2e-2 abs/rel, logsumexp within 2e-3), an
 fused append, by reading the pool back: the block's rows land in the pages the table names,
 bit for bit, and nothing else changes."""
 
-import contextlib
 import math
-import os
 
 import numpy as np
 import pytest
@@ -25,22 +23,6 @@ LSE_TOL = dict(rtol=2e-3, atol=2e-3)
 
 def host(t):
     return t.detach().float().cpu().numpy()
-
-
-@contextlib.contextmanager
-def single_role_kernel():
-    """The paged entry runs on the single-role attention kernel; the dense entries default to the
-    producer/consumer kernel, which deals tiles to splits in another order (same mathematics, another
-    rounding of the last bit).  Byte-for-byte comparisons therefore pin the dense call to the same kernel."""
-    old = os.environ.get("DFLASH_SDPA_PRODUCERS")
-    os.environ["DFLASH_SDPA_PRODUCERS"] = "0"
-    try:
-        yield
-    finally:
-        if old is None:
-            del os.environ["DFLASH_SDPA_PRODUCERS"]
-        else:
-            os.environ["DFLASH_SDPA_PRODUCERS"] = old
 
 
 def paged_case(seed, B, Hq, Hk, lengths, D, page_size, dtype=torch.bfloat16, spare_pages=3, head_pad=0, page_pad=0):
@@ -94,8 +76,7 @@ def test_paged_equals_dense_and_oracle(gpu_lib, cfg, dtype):
     N = L + 16
     q, k, v, k_pool, v_pool, table = paged_case(L + P, B, Hq, Hk, [N] * B, D, P, dtype)
     scale = 1.0 / math.sqrt(D)
-    with single_role_kernel():
-        want, want_lse = K.batched_sdpa_2pass(q, k, v, scale, return_lse=True)
+    want, want_lse = K.batched_sdpa_2pass(q, k, v, scale, return_lse=True)
     got, got_lse = K.batched_sdpa_2pass_paged(q, k_pool, v_pool, table, scale, N, return_lse=True)
     torch.cuda.synchronize()
     assert torch.equal(got, want) and torch.equal(got_lse, want_lse)
@@ -116,8 +97,7 @@ def test_paged_padded_pitches_and_ragged_lengths(gpu_lib):
     lens = [116, 349, 666]
     q, k, v, k_pool, v_pool, table = paged_case(3, B, Hq, Hk, lens, D, P, head_pad=64, page_pad=128)
     kv_len = torch.tensor(lens, dtype=torch.int32, device="cuda")
-    with single_role_kernel():
-        want = K.batched_sdpa_2pass(q, k, v, 1.0 / 16, kv_len=kv_len)
+    want = K.batched_sdpa_2pass(q, k, v, 1.0 / 16, kv_len=kv_len)
     got = K.batched_sdpa_2pass_paged(q, k_pool, v_pool, table, 1.0 / 16, max(lens), lengths=kv_len)
     assert torch.equal(got, want)
     for b in range(B):                             # each sequence against the oracle on its own keys
@@ -147,8 +127,7 @@ def test_paged_fused_append(gpu_lib, cfg):
             k_pool[tb[b, n // P], :, n % P] = 5.0
             v_pool[tb[b, n // P], :, n % P] = 5.0
     scale = 1.0 / math.sqrt(D)
-    with single_role_kernel():
-        want, want_lse = K.batched_sdpa_2pass(q, k, v, scale, return_lse=True)
+    want, want_lse = K.batched_sdpa_2pass(q, k, v, scale, return_lse=True)
     got, got_lse = K.batched_sdpa_2pass_paged(q, k_pool, v_pool, table, scale, N, k_new=k_new, v_new=v_new, return_lse=True)
     torch.cuda.synchronize()
     assert torch.equal(got, want) and torch.equal(got_lse, want_lse)
@@ -175,8 +154,7 @@ def test_paged_fused_append_ragged_device_lengths(gpu_lib):
             v_pool[tb[b, n // P], :, n % P] = 9.0
     kv_len = torch.tensor(lens, dtype=torch.int32, device="cuda")
     cache_len = torch.tensor(Ls, dtype=torch.int32, device="cuda")
-    with single_role_kernel():
-        want = K.batched_sdpa_2pass(q, k, v, 1.0 / 16, kv_len=kv_len)
+    want = K.batched_sdpa_2pass(q, k, v, 1.0 / 16, kv_len=kv_len)
     got = K.batched_sdpa_2pass_paged(q, k_pool, v_pool, table, 1.0 / 16, max(lens), k_new=k_new, v_new=v_new, lengths=cache_len)
     assert torch.equal(got, want)
     # rows beyond a sequence's own length in its last page are not compared: they were never defined
@@ -192,8 +170,7 @@ def test_paged_long_context_equals_dense(gpu_lib):
 
     B, Hq, Hk, L, D, P = 1, 16, 2, 32768, 256, 256
     q, k, v, k_pool, v_pool, table = paged_case(2, B, Hq, Hk, [L + 16], D, P)
-    with single_role_kernel():
-        want, want_lse = K.batched_sdpa_2pass(q, k, v, 1.0 / 16, return_lse=True)
+    want, want_lse = K.batched_sdpa_2pass(q, k, v, 1.0 / 16, return_lse=True)
     got, got_lse = K.batched_sdpa_2pass_paged(q, k_pool, v_pool, table, 1.0 / 16, L + 16, return_lse=True)
     assert torch.equal(got, want) and torch.equal(got_lse, want_lse)
 
@@ -268,8 +245,7 @@ def test_paged_random_shapes(gpu_lib, seed):
                                                     head_pad=int(rng.choice([0, 8, 64])), page_pad=int(rng.choice([0, 16])))
         scale = 1.0 / math.sqrt(D)
         kv_len = torch.tensor(lens, dtype=torch.int32, device="cuda")
-        with single_role_kernel():
-            want, want_lse = K.batched_sdpa_2pass(q, k, v, scale, return_lse=True, kv_len=kv_len)
+        want, want_lse = K.batched_sdpa_2pass(q, k, v, scale, return_lse=True, kv_len=kv_len)
         if append:
             k_new = torch.stack([k[b, :, Ls[b]:Ls[b] + 16] for b in range(B)]).contiguous()
             v_new = torch.stack([v[b, :, Ls[b]:Ls[b] + 16] for b in range(B)]).contiguous()
