@@ -209,6 +209,26 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
     const int b = blockIdx.z;
     const int hcount = (A.G - hg0) < kHeadsPerWG ? (A.G - hg0) : kHeadsPerWG;
 
+    // Paged: each producer wave keeps the page-table entries of this workgroup's next 64 tiles in a register, one
+    // tile per lane (a single gather, so a cold table costs one round trip per 64 tiles and none inside the loop),
+    // and the 64 after those in a second register that is fetched a whole batch ahead.  The first gather is issued
+    // here, ahead of the device-side length, so that the two cold reads overlap; it therefore covers the tiles of
+    // the host-side bound N, which the table spans by contract.
+    int ent_cur = 0, ent_nxt = 0, ent_base = 0;
+    auto load_entries = [&](int base) -> int {
+        // no branch and no arithmetic on the value here: the wait for it then sits at its first use, not at the load
+        const int nt_max = (A.N + kBN - 1) / kBN;
+        int tile = split + (base + lane) * A.S;
+        tile = tile < nt_max ? tile : nt_max - 1;
+        return A.page_table[(size_t)b * A.table_stride + ((tile * kBN) >> A.page_shift)];
+    };
+    if constexpr (PAGED) {
+        if (producer) {
+            ent_cur = load_entries(0);
+            ent_nxt = load_entries(64);
+        }
+    }
+
     int Nb = A.kv_len_dev ? A.kv_len_dev[b] + A.len_bias : A.N;
     Nb = Nb < kM ? kM : (Nb > A.N ? A.N : Nb);
     const int nt = (Nb + kBN - 1) / kBN;
@@ -234,8 +254,9 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
                                   : ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
     const unsigned char* kbase = reinterpret_cast<const unsigned char*>(A.k) + head_off;
     const unsigned char* vbase = reinterpret_cast<const unsigned char*>(A.v) + head_off;
-    // Byte offset of key n's row from kbase / vbase (the K and V pools share one layout).  Paged: the page comes
-    // from the table, clamped to the pool; a tile never straddles a page (page sizes are multiples of kBN).
+    // Byte offset of key n's row from kbase / vbase (the K and V pools share one layout), for the rows that are
+    // looked up one by one: those of the fused append.  Paged: the page comes from the table, clamped to the pool.
+    // (Tiles take tile_off() below; a tile never straddles a page, page sizes being multiples of kBN.)
     const int page_mask = PAGED ? (1 << A.page_shift) - 1 : 0;
     auto row_off = [&](int key) -> size_t {
         if constexpr (PAGED) {
@@ -248,14 +269,16 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
     };
     // Fused append: keys Nb-16 .. Nb-1 are read from k_new / v_new, and one workgroup per KV head stores them
     // into the cache rows they stand for (paged: the 16 rows may straddle a page, so every row looks its page up).
+    // The copy is done by the compute waves, which have nothing to do until the first tile lands, of the LAST split,
+    // which never holds more tiles than the others: it stays off the launch's critical path.
     const bool fused = A.k_new != nullptr;
     const int cache_rows = fused ? Nb - kM : Nb;       // keys below this index are read from the cache
     const unsigned char* knew = reinterpret_cast<const unsigned char*>(A.k_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
     const unsigned char* vnew = reinterpret_cast<const unsigned char*>(A.v_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
-    if (fused && A.k_cache && split == 0 && hg0 == 0) {
+    if (fused && A.k_cache && split == A.S - 1 && hg0 == 0 && !producer) {
         const u32x4_t* ksrc = reinterpret_cast<const u32x4_t*>(knew);
         const u32x4_t* vsrc = reinterpret_cast<const u32x4_t*>(vnew);
-        for (int i = tid; i < kM * L::CPR; i += kPartialThreads) {
+        for (int i = tid; i < kM * L::CPR; i += 4 * 64) {
             const size_t off = head_off + row_off(cache_rows + i / L::CPR) + (size_t)(i % L::CPR) * 16;
             *reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.k_cache) + off) = ksrc[i];
             *reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.v_cache) + off) = vsrc[i];
@@ -288,7 +311,8 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
                 }
             } else {
                 // Tail tile: rows past the end re-read the last key (masked later); with a fused append the
-                // block's own 16 rows are taken from k_new / v_new instead of the cache.
+                // block's own 16 rows are taken from k_new / v_new instead of the cache.  Its cache rows sit behind
+                // the tile's own offset like any other tile's (paged: a tile lies in one page).
 #pragma unroll
                 for (int j = 0; j < L::LPP; ++j) {
                     const int rg = (2 * j + pw) * L::RPI;
@@ -297,7 +321,8 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
                     key = key < Nb ? key : Nb - 1;
                     const uint32_t sw = k_swizzle ? (uint32_t)((ld_pos ^ (row & 15)) * 16) : (uint32_t)((ld_pos ^ (4 * (row & 3))) * 16);
                     const unsigned char* nw = is_k ? knew : vnew;
-                    const unsigned char* src = key < cache_rows ? base + row_off(key) : nw + (size_t)(key - cache_rows) * L::ROWB;
+                    const unsigned char* src = key < cache_rows ? base + toff + (size_t)(key - key0) * L::ROWB
+                                                                : nw + (size_t)(key - cache_rows) * L::ROWB;
                     async_load_16B_addr(src + sw, lds_tile + rg * L::ROWB);
                 }
             }
@@ -308,12 +333,30 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
         auto issue_v = [&](int t, size_t toff) {
             if (t < t_end) issue_rows(vbase, false, t, toff, smem_lds + L::V_RING + ((t - t_begin) % kRingSlots) * L::KT, false);
         };
-        // Offset of tile t's first row (a wave-uniform value; paged: one scalar read of the page table).  Inside the
-        // loop it is looked up an iteration before it is used, so the table read never delays a request.
-        auto tile_off = [&](int t) -> size_t { return t < t_end ? row_off(key_of(t)) : 0; };
+        // Offset of tile t's first row (a wave-uniform value); paged: from the entries gathered at the top of the
+        // kernel, refilled a batch ahead.  Tiles are asked for in increasing order.
+        auto tile_off = [&](int t) -> size_t {
+            if (t >= t_end) return 0;
+            if constexpr (PAGED) {
+                if (t - ent_base >= 64) {                                        // uniform
+                    ent_cur = ent_nxt;
+                    ent_base += 64;
+                    ent_nxt = load_entries(ent_base + 64);
+                    // Take the value here, once per 64 tiles.  Left pending, the compiler carries the load across the
+                    // loop and puts a vmcnt(0) in front of every iteration's use, which drains the tile requests too.
+                    asm volatile("" : "+v"(ent_nxt));
+                }
+                int e = __builtin_amdgcn_readlane(ent_cur, (t - ent_base) & 63);
+                e = e < 0 ? 0 : (e >= A.num_pages ? A.num_pages - 1 : e);      // a stale table cannot leave the pool
+                return (size_t)e * (size_t)A.kv_batch_stride * 2 + (size_t)(key_of(t) & page_mask) * L::ROWB;
+            } else {
+                return (size_t)key_of(t) * L::ROWB;
+            }
+        };
         // loads of group t still outstanding when one waits for the group before it
         auto group_loads = [&](int t) { return (t < t_end ? L::LPP : 0) + (t + 1 < t_end ? L::LPP : 0); };
 
+        if constexpr (PAGED) asm volatile("" : "+v"(ent_cur), "+v"(ent_nxt));   // both gathers have landed from here on
         {
             const size_t o0 = tile_off(t_begin), o1 = tile_off(t_begin + 1);
             issue_k(t_begin, o0);

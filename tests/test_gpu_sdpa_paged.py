@@ -175,6 +175,26 @@ def test_paged_long_context_equals_dense(gpu_lib):
     assert torch.equal(got, want) and torch.equal(got_lse, want_lse)
 
 
+def test_paged_many_tiles_per_workgroup_equals_dense(gpu_lib):
+    """A batch wide enough that the key axis is split only 8 ways: every workgroup walks 150 tiles, so the
+    producers' per-lane store of page entries (64 tiles a batch) is refilled twice."""
+    from swiftlm_amd import DFlashKernels as K
+
+    B, Hq, Hk, L, D, P = 16, 2, 2, 38400, 128, 64
+    q, k, v, k_pool, v_pool, table = paged_case(6, B, Hq, Hk, [L + 16] * B, D, P)
+    scale = 1.0 / math.sqrt(D)
+    want, want_lse = K.batched_sdpa_2pass(q, k, v, scale, return_lse=True)
+    got, got_lse = K.batched_sdpa_2pass_paged(q, k_pool, v_pool, table, scale, L + 16, return_lse=True)
+    assert torch.equal(got, want) and torch.equal(got_lse, want_lse)
+    # and the dense result itself against plain fp32 attention on one sequence
+    b = 5
+    s = torch.einsum("hmd,hnd->hmn", q[b].float() * scale, k[b].float())
+    n = L + 16
+    vis = torch.arange(n, device="cuda")[None, :] <= (n - 16 + torch.arange(16, device="cuda"))[:, None]
+    ref = torch.einsum("hmn,hnd->hmd", torch.softmax(s.masked_fill(~vis, float("-inf")), -1), v[b].float())
+    np.testing.assert_allclose(host(got[b]), host(ref), rtol=2e-2, atol=2e-2)
+
+
 def test_paged_out_of_range_table_entries_stay_inside_the_pool(gpu_lib):
     """Entries outside [0, num_pages) are clamped on the device: the call completes and equals the
     call with the clamped table."""
