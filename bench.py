@@ -225,14 +225,24 @@ def main():
         if cc - 1 < T - 1:
             p[cc - 1] = row[cc] + 1                # first mismatch -> acceptance length cc - 1
         ids[s], post[s] = row, p
-    ids_d, post_d = ids.cuda(), post.cuda()
+    # [step, ids | posterior, T]: one device-to-device copy hands a step its token ids (what the drafter and the
+    # target's argmax would leave on the device), two consecutive steps' worth when a graph holds two steps
+    staged_d = torch.stack([ids, post], dim=1).cuda()
     step_no = [0]
 
     def stage(phase):
         s = step_no[0]
-        stack.verify_ids[phase].copy_(ids_d[s], non_blocking=True)
-        stack.posterior[phase].copy_(post_d[s], non_blocking=True)
+        stack.accept_inputs[phase].copy_(staged_d[s], non_blocking=True)
         step_no[0] += 1
+
+    def stage_pair(phase):
+        s = step_no[0]
+        if phase == 0:
+            stack.accept_inputs.copy_(staged_d[s:s + 2], non_blocking=True)
+        else:
+            stage(phase); stage(1 - phase)
+            return
+        step_no[0] += 2
 
     def eager_step(before_launch=None):
         stage(stack.phase)
@@ -264,7 +274,7 @@ def main():
         for _ in range(n_steps // 2):
             if graphs is not None:
                 ph = stack.phase
-                stage(ph); stage(1 - ph)
+                stage_pair(ph)
                 graphs[ph].replay()
             else:
                 eager_step(); eager_step()

@@ -124,8 +124,10 @@ class HybridVerifyStack:
         self.offset = torch.tensor([cfg.context], dtype=torch.int32, device=device)
         self.accept = torch.zeros(4, dtype=torch.int32, device=device)
         # acceptance inputs of the step being enqueued, one pair per ping-pong phase
-        self.verify_ids = [torch.zeros(T, dtype=torch.int32, device=device) for _ in range(2)]
-        self.posterior = [torch.zeros(T, dtype=torch.int32, device=device) for _ in range(2)]
+        # (one block [phase, ids | posterior, T], so that a caller can hand over both phases with a single copy)
+        self.accept_inputs = torch.zeros(2, 2, T, dtype=torch.int32, device=device)
+        self.verify_ids = [self.accept_inputs[ph, 0] for ph in range(2)]
+        self.posterior = [self.accept_inputs[ph, 1] for ph in range(2)]
         self.phase = 0               # which state buffer holds the pre-verify state
         # host pointer tables for the batched replay, one per phase
         self._tables = []
