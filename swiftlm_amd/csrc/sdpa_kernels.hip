@@ -110,8 +110,11 @@ typedef __attribute__((ext_vector_type(8))) short s16x8_t;
 // travels in M0).  Issued as inline assembly on purpose: the compiler then does not track these
 // loads, so it cannot force a full vmcnt(0) drain ahead of every LDS read or barrier; completion
 // is tracked by hand with wait_vmcnt<> below, which is what keeps several tiles in flight.
+// K/V rows are read once per call, so their loads carry the non-temporal hint: the stream (800 MB per verify step
+// at the benchmark's shape) then no longer pushes the recurrent state, the tapes and the split partials out of
+// the 256 MB memory-side cache -- worth 8 % of the whole step, most of it in the OTHER kernels.
 __device__ __forceinline__ void async_load_16B(const unsigned char* gbase, uint32_t goff, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt"
                  :
                  : "v"(goff), "s"(gbase), "s"(__builtin_amdgcn_readfirstlane(lds_base))
                  : "memory", "m0");
@@ -125,12 +128,19 @@ __device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char*
     return (const unsigned char*)(((uint64_t)hi << 32) | lo);
 }
 
-// Same, with a full per-lane 64-bit address (rows that come from different buffers).
-__device__ __forceinline__ void async_load_16B_addr(const unsigned char* gptr, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                 :
-                 : "v"((uint64_t)gptr), "s"(__builtin_amdgcn_readfirstlane(lds_base))
-                 : "memory", "m0");
+// Same, with a full per-lane 64-bit address (rows that come from different buffers).  STREAM: non-temporal, for
+// K/V rows; Q, which every workgroup of the head re-reads, is loaded without the hint.
+template <bool STREAM> __device__ __forceinline__ void async_load_16B_addr(const unsigned char* gptr, uint32_t lds_base) {
+    if constexpr (STREAM)
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt"
+                     :
+                     : "v"((uint64_t)gptr), "s"(__builtin_amdgcn_readfirstlane(lds_base))
+                     : "memory", "m0");
+    else
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                     :
+                     : "v"((uint64_t)gptr), "s"(__builtin_amdgcn_readfirstlane(lds_base))
+                     : "memory", "m0");
 }
 
 // s_waitcnt vmcnt(n) only (expcnt and lgkmcnt left alone), GFX9 encoding.
@@ -323,7 +333,7 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
                     const unsigned char* nw = is_k ? knew : vnew;
                     const unsigned char* src = key < cache_rows ? base + toff + (size_t)(key - key0) * L::ROWB
                                                                 : nw + (size_t)(key - cache_rows) * L::ROWB;
-                    async_load_16B_addr(src + sw, lds_tile + rg * L::ROWB);
+                    async_load_16B_addr<true>(src + sw, lds_tile + rg * L::ROWB);
                 }
             }
         };
@@ -370,7 +380,7 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
                 for (int j = 0; j < L::QPP; ++j) {
                     const int row = (2 * j + pw) * L::RPI + ld_rsub;           // 0..127 over the four compute waves
                     const int head = (row >> 4) < hcount ? (row >> 4) : 0;
-                    async_load_16B_addr(qb + (size_t)(head * kM + (row & 15)) * L::ROWB + ((ld_pos ^ (row & 15)) * 16),
+                    async_load_16B_addr<false>(qb + (size_t)(head * kM + (row & 15)) * L::ROWB + ((ld_pos ^ (row & 15)) * 16),
                                         smem_lds + (2 * j + pw) * L::RPI * L::ROWB);
                 }
             }
