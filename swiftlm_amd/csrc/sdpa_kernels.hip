@@ -21,9 +21,9 @@
 // The same trick gives O^T = V^T P^T, whose accumulators are again one query row
 // per lane, so the running rescale is a per-lane scalar.  P^T is taken straight
 // from the S^T accumulators: the 8 k-elements a lane feeds to the second MFMA are
-// whatever keys its accumulators hold, and V^T is laid out in LDS in that same
-// key order (bits 2 and 3 of the key index swapped), which is legal because a
-// contraction may enumerate its index in any order.
+// whatever keys its accumulators hold, and the V^T operand is gathered from LDS
+// in that same key order (two transposing reads of four keys each), which is
+// legal because a contraction may enumerate its index in any order.
 //
 // Semantics follow Sources/DFlash/DFlashKernels.swift:737-815 (entry), :563-649
 // (partials: causal rule :614, GQA mapping :575) and :661-720 (combine).
