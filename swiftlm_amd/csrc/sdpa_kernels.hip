@@ -738,7 +738,7 @@ template <typename Tag, int D>
 __global__ __launch_bounds__(kCombineThreads) void sdpa_combine_kernel(CombineArgs A) {
     constexpr int TPG = D / 8;                     // threads spanning one row, 8 elements (16 B) each
     constexpr int NG = kCombineThreads / TPG;         // split groups walking the partials in parallel
-    constexpr int UNROLL = 4;
+    constexpr int UNROLL = 16;                     // row loads in flight per thread: one round trip for S <= 16 * NG
     __shared__ float w_s[kMaxSplits];
     __shared__ float red_s[kCombineThreads / 64];
     __shared__ float acc_s[NG][D];
@@ -782,13 +782,15 @@ __global__ __launch_bounds__(kCombineThreads) void sdpa_combine_kernel(CombineAr
         for (int u = 0; u < UNROLL; ++u) {
             const int s = s0 + u * NG;
             w[u] = s < A.S ? w_s[s] : 0.f;
-            raw[u] = u32x4_t{0u, 0u, 0u, 0u};
-            if (w[u] != 0.f) raw[u] = *reinterpret_cast<const u32x4_t*>(po + (size_t)s * gridDim.x * D);   // empty splits hold no data
+            // Loaded without looking at the weight (a branch per load makes the loads wait for one another); the rows of
+            // empty splits hold no data, whatever was read from them is dropped below.
+            raw[u] = *reinterpret_cast<const u32x4_t*>(po + (size_t)(s < A.S ? s : 0) * gridDim.x * D);
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
+                if (w[u] == 0.f) raw[u][e] = 0u;
                 acc[2 * e] = fmaf(w[u], Tag::to_f32((uint16_t)(raw[u][e] & 0xffffu)), acc[2 * e]);
                 acc[2 * e + 1] = fmaf(w[u], Tag::to_f32((uint16_t)(raw[u][e] >> 16)), acc[2 * e + 1]);
             }
