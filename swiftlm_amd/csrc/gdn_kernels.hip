@@ -67,7 +67,7 @@ struct ReplayArgs {
     int T_tape, Hk, Hv, Dv;
 };
 
-constexpr int kReplayChunk = 32;  // steps staged in LDS at a time (16 for Dk = 256)
+constexpr int kReplayChunk = 16;  // steps staged in LDS at a time (8 for Dk = 256): one chunk covers the 16-token verify block
 
 // One thread owns 4 consecutive key channels of NR state rows.  DK/4 threads
 // span a row, so a 256-thread workgroup covers RPP = floor(1024/DK) rows per pass
@@ -118,7 +118,8 @@ __global__ __launch_bounds__(kThreads) void tape_replay_kernel(ReplayBatch P, Re
         __syncthreads();
         n = n_s;
     } else {
-        n = A.steps_dev ? *A.steps_dev : A.steps;
+        n = A.steps;
+        if (A.steps_dev) n = __builtin_amdgcn_readfirstlane(*A.steps_dev);   // (kept a branch: as a select of two addresses the host-side count lands in scratch)
     }
     n = n < 0 ? 0 : (n > A.T_tape ? A.T_tape : n);
     if (A.skip_if_full && n == A.T_tape) return;   // uniform over the grid
@@ -129,33 +130,109 @@ __global__ __launch_bounds__(kThreads) void tape_replay_kernel(ReplayBatch P, Re
     const void* kk = P.k[layer];
     const void* gg = P.g[layer];
 
+    // ---- loads ----
+    // A chunk's operands are requested as raw bits, array by array, inside branches that hold nothing but loads,
+    // and converted only after the last request has gone out; the state rows are requested in between.  (With a
+    // conversion or an LDS store next to each load, the compiler waits for every load before it issues the next:
+    // half a dozen dependent round trips per workgroup.)  Addresses are clamped instead of predicated, values that
+    // must not count are dropped at the LDS store.
+    constexpr int KI = (TC * TPR + kThreads - 1) / kThreads;      // k (and vector gate) groups of 4 per thread
+    constexpr int DI = (TC * ROWS + kThreads - 1) / kThreads;     // tape values per thread
+    const bool in32 = A.in_dtype == DFLASH_F32, tape32 = A.tape_dtype == DFLASH_F32;
+    const bool in_bf16 = A.in_dtype == DFLASH_BF16, tape_bf16 = A.tape_dtype == DFLASH_BF16;
+    uint4 k32[KI], g32[VEC_G ? KI : 1];
+    uint2 k16[KI], g16[VEC_G ? KI : 1];
+    float d32[DI], gs32;
+    uint32_t d16[DI], gs16;                                   // 16-bit values, zero-extended
+    int on_r;
+    auto cvt16 = [](uint16_t bits, bool is_bf16) -> float {
+        return is_bf16 ? __uint_as_float(((uint32_t)bits) << 16) : (float)__builtin_bit_cast(_Float16, bits);
+    };
+    auto cvt4 = [&](uint4 w, uint2 h) -> float4 {
+        if (in32) return make_float4(__uint_as_float(w.x), __uint_as_float(w.y), __uint_as_float(w.z), __uint_as_float(w.w));
+        return make_float4(cvt16((uint16_t)(h.x & 0xffffu), in_bf16), cvt16((uint16_t)(h.x >> 16), in_bf16),
+                           cvt16((uint16_t)(h.y & 0xffffu), in_bf16), cvt16((uint16_t)(h.y >> 16), in_bf16));
+    };
+    auto request_chunk = [&](int t0, int tc) {
+        size_t kidx[KI], gidx[KI], didx[DI];
+#pragma unroll
+        for (int u = 0; u < KI; ++u) {
+            const int i = tid + u * kThreads, c = (i % TPR) * 4;
+            const int t = (i / TPR) < tc ? (i / TPR) : tc - 1;
+            const size_t bt = (size_t)b * A.T_tape + t0 + t;
+            kidx[u] = (bt * A.Hk + hk) * DK + c;
+            gidx[u] = (bt * A.Hv + hv) * DK + c;
+        }
+#pragma unroll
+        for (int u = 0; u < DI; ++u) {
+            const int i = tid + u * kThreads, r = i % ROWS;
+            const int t = (i / ROWS) < tc ? (i / ROWS) : tc - 1;
+            const int row = (row0 + r) < A.Dv ? row0 + r : A.Dv - 1;
+            didx[u] = (((size_t)b * A.T_tape + t0 + t) * A.Hv + hv) * A.Dv + row;
+        }
+        const int tl = tid < tc ? tid : tc - 1;
+        const size_t bts = (size_t)b * A.T_tape + t0 + tl;
+        if (in32) {
+#pragma unroll
+            for (int u = 0; u < KI; ++u) {
+                k32[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const float*>(kk) + kidx[u]);
+                if (VEC_G) g32[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const float*>(gg) + gidx[u]);
+            }
+            if (!VEC_G) gs32 = reinterpret_cast<const float*>(gg)[bts * A.Hv + hv];
+        } else {
+#pragma unroll
+            for (int u = 0; u < KI; ++u) {
+                k16[u] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(kk) + kidx[u]);
+                if (VEC_G) g16[u] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(gg) + gidx[u]);
+            }
+            if (!VEC_G) gs16 = reinterpret_cast<const uint16_t*>(gg)[bts * A.Hv + hv];
+        }
+        if (tape32) {
+#pragma unroll
+            for (int u = 0; u < DI; ++u) d32[u] = reinterpret_cast<const float*>(tape)[didx[u]];
+        } else {
+#pragma unroll
+            for (int u = 0; u < DI; ++u) d16[u] = reinterpret_cast<const uint16_t*>(tape)[didx[u]];
+        }
+        on_r = A.mask ? (int)mask_on(A.mask, A.mask_dtype, (int)bts) : 1;
+    };
+    auto park_chunk = [&](int tc) {
+#pragma unroll
+        for (int u = 0; u < KI; ++u) {
+            const int i = tid + u * kThreads, t = i / TPR, c = (i % TPR) * 4;
+            if (t < tc) {
+                store4(&k_s[t][c], cvt4(k32[u], k16[u]));
+                if (VEC_G) store4(&g_s[t][c], cvt4(g32[VEC_G ? u : 0], g16[VEC_G ? u : 0]));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < DI; ++u) {
+            const int i = tid + u * kThreads, t = i / ROWS, r = i % ROWS;
+            if (t < tc) d_s[t][r] = (row0 + r) < A.Dv ? (tape32 ? d32[u] : cvt16((uint16_t)d16[u], tape_bf16)) : 0.f;
+        }
+        if (tid < tc) {
+            if (!VEC_G) g_s[0][tid] = in32 ? gs32 : cvt16((uint16_t)gs16, in_bf16);
+            on_s[tid] = on_r;
+        }
+    };
+
+    const int tc0 = n < TC ? n : TC;
+    if (n > 0) request_chunk(0, tc0);
     float4 s[NR];
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
-        const int r = row0 + rsub + RPP * i;
-        s[i] = (owner && r < A.Dv) ? load4(s_in + (size_t)r * DK + c4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        int r = row0 + rsub + RPP * i;
+        r = r < A.Dv ? r : A.Dv - 1;                       // clamped: rows outside are never stored
+        s[i] = load4(s_in + (size_t)r * DK + c4);
     }
 
     for (int t0 = 0; t0 < n; t0 += TC) {
         const int tc = (n - t0) < TC ? (n - t0) : TC;
-        if (t0) __syncthreads();
-        // ---- stage this chunk's operands as float ----
-        for (int i = tid; i < tc * TPR; i += kThreads) {
-            const int t = i / TPR, c = (i % TPR) * 4;
-            const size_t bt = (size_t)b * A.T_tape + t0 + t;
-            store4(&k_s[t][c], load4_rt(kk, A.in_dtype, (bt * A.Hk + hk) * DK + c));
-            if (VEC_G) store4(&g_s[t][c], load4_rt(gg, A.in_dtype, (bt * A.Hv + hv) * DK + c));
+        if (t0) {
+            __syncthreads();
+            request_chunk(t0, tc);
         }
-        for (int i = tid; i < tc * ROWS; i += kThreads) {
-            const int t = i / ROWS, r = i % ROWS;
-            const size_t bt = (size_t)b * A.T_tape + t0 + t;
-            d_s[t][r] = (row0 + r) < A.Dv ? load1_rt(tape, A.tape_dtype, (bt * A.Hv + hv) * A.Dv + row0 + r) : 0.f;
-        }
-        if (tid < tc) {
-            const size_t bt = (size_t)b * A.T_tape + t0 + tid;
-            if (!VEC_G) g_s[0][tid] = load1_rt(gg, A.in_dtype, bt * A.Hv + hv);
-            on_s[tid] = A.mask ? (int)mask_on(A.mask, A.mask_dtype, (int)bt) : 1;
-        }
+        park_chunk(tc);
         __syncthreads();
         // ---- serial steps, operands from LDS ----
         for (int t = 0; t < tc; ++t) {
