@@ -322,11 +322,14 @@ def main():
     sdpa_bytes = stack.sdpa_bytes(kv_mid)
     achieved = sdpa_bytes / (sdpa_us * 1e-6) / 1e9
 
+    # counter-measured bytes per launch: only for the workload the counters were collected on
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "sdpa_partial_traffic.json")
-    if os.path.exists(tpath):
+    if os.path.exists(tpath) and args.context == 32768 and not args.page_size:
         try:
-            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+            tj = json.load(open(tpath))
+            if tj.get("workload") == "config4 L=32768":
+                traffic = tj.get("hbm_bytes_per_launch")
         except Exception:
             traffic = None
 
