@@ -98,6 +98,23 @@ def test_sdpa_config2_against_c_oracle(gpu_lib):
     assert torch.equal(out2, out)
 
 
+@pytest.mark.parametrize("cfg", [(1, 8, 1, 40000, 256), (1, 4, 1, 40000, 128), (1, 1, 1, 70000, 256)],
+                         ids=lambda c: f"Hq{c[1]}_Hk{c[2]}_L{c[3]}_D{c[4]}")
+def test_sdpa_single_kv_head_uses_every_split(gpu_lib, cfg):
+    """One KV head and one batch: the key axis is cut into as many splits as the GPU has CUs (256 on the
+    benchmark's GPU), so the combine kernel walks its partials in more than one pass, and with Hq = 1 most of
+    a workgroup's query rows are absent.  Checked against a float32 restatement, logsumexp included."""
+    from swiftlm_amd import DFlashKernels as K
+
+    B, Hq, Hk, L, D = cfg
+    q, k, v = gpu_inputs(L + 11, B, Hq, Hk, L, D)
+    scale = 1.0 / math.sqrt(D)
+    out, lse = K.batched_sdpa_2pass(q, k, v, scale, return_lse=True)
+    ow, lw = torch_reference(q, k, v, scale)
+    np.testing.assert_allclose(host(out), host(ow), **OUT_TOL)
+    np.testing.assert_allclose(host(lse), host(lw), **LSE_TOL)
+
+
 @pytest.mark.parametrize("L", [32768, 40960, 102400])
 def test_sdpa_long_context_properties(gpu_lib, L):
     """Benchmark configuration 3 sizes.  Properties that do not need a CPU pass: constant V gives
