@@ -137,6 +137,10 @@ def gated_delta_ops_with_tape(q, k, v, g, beta, state, mask=None, *, dtype=np.fl
     ``S = S' + k (x) delta``; ``y = sum_dk S*q``.  A masked step keeps S and
     emits y = 0 and delta = 0 (:446-453).
 
+    ``requant`` ('bf16' | 'f16') follows the Metal kernel for a low-precision state
+    (:148-199): the state is re-rounded to the storage type after every executed step
+    (:183-186), while that step's y is read from the state before the rounding (:171-172).
+
     Returns (y [B,T,Hv,Dv], state [B,Hv,Dv,Dk], tape [B,T,Hv,Dv] float32).
     """
     q = np.asarray(q, dtype=dtype)
@@ -159,8 +163,11 @@ def gated_delta_ops_with_tape(q, k, v, g, beta, state, mask=None, *, dtype=np.fl
         kt = k[:, t, :, None, :]
         kv_mem = (decayed * kt).sum(axis=-1)
         delta = (v[:, t] - kv_mem) * beta[:, t, :, None]
-        new_state = quantize(decayed + kt * delta[..., None], requant)
-        y = (new_state * q[:, t, :, None, :]).sum(axis=-1)
+        updated = decayed + kt * delta[..., None]
+        # The Metal kernel reads y out of the updated state BEFORE it re-rounds that state to the
+        # storage type (DFlashKernels.swift:171-172, rounding at :183-186); without requant the two coincide.
+        y = (updated * q[:, t, :, None, :]).sum(axis=-1)
+        new_state = quantize(updated, requant)
         if mask is not None:
             step = np.asarray(mask)[:, t] > 0.5
             sg = step[:, None, None, None]

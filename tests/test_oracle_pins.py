@@ -184,6 +184,40 @@ def test_gated_delta_matches_kimi_restatement():
     np.testing.assert_allclose(S, s, rtol=1e-12, atol=1e-14)
 
 
+def test_forward_low_precision_state_rounds_state_not_y():
+    """One step by hand (DFlashKernels.swift:148-199 with a bf16 state): the stored state is the
+    bf16 rounding of the updated state (:183-186) while y is read from the state before that
+    rounding (:171-172).  Values are picked so that the two differ: 1 + 2^-9 is not a bf16 number."""
+    eps = 2.0 ** -9
+    S0 = np.array([[[[1.0, 0.0]]]], np.float32)            # one head, one row, Dk = 2
+    k = np.array([[[[0.0, 1.0]]]], np.float32)
+    q = np.array([[[[1.0, 1.0]]]], np.float32)
+    v = np.array([[[[eps]]]], np.float32)
+    g = np.ones((1, 1, 1), np.float32)
+    beta = np.ones((1, 1, 1), np.float32)
+    # by hand: S' = S0; m = S'k = 0; delta = (eps - 0) * 1 = eps; S = [1, eps]; y = S q = 1 + eps
+    y, S, tape = O.gated_delta_ops_with_tape(q, k, v, g, beta, S0, requant="bf16")
+    assert tape[0, 0, 0, 0] == np.float32(eps)
+    assert y[0, 0, 0, 0] == np.float32(1.0 + eps)          # not re-rounded: bf16 would give 1.0
+    np.testing.assert_array_equal(S[0, 0, 0], [1.0, eps])  # both entries are bf16 numbers
+    # second step: now the update lands on the SAME entry, so the state must round and y must not
+    k2 = np.array([[[[1.0, 0.0]]], [[[1.0, 0.0]]]], np.float32).reshape(1, 2, 1, 2)
+    q2 = np.tile(q, (1, 2, 1, 1))
+    v2 = np.array([1.0, 1.0 + 2 * eps + eps], np.float32).reshape(1, 2, 1, 1)   # step 2: delta = v - S[0]
+    S1 = np.array([[[[1.0, 0.0]]]], np.float32)
+    y2, S2, t2 = O.gated_delta_ops_with_tape(q2, k2, v2, np.ones((1, 2, 1), np.float32),
+                                             np.ones((1, 2, 1), np.float32), S1, requant="bf16")
+    # step 1: m = 1, delta = 0, S = [1, 0]; step 2: m = 1, delta = 3 eps, S = [1 + 3 eps, 0] -> y = 1 + 3 eps,
+    # stored state rounds 1 + 3*2^-9 (= 1.005859375) to the bf16 grid {1, 1 + 2^-7}: nearest is 1 + 2^-7
+    assert t2[0, 1, 0, 0] == np.float32(3 * eps)
+    assert y2[0, 1, 0, 0] == np.float32(1.0 + 3 * eps)
+    np.testing.assert_array_equal(S2[0, 0, 0], [1.0 + 2.0 ** -7, 0.0])
+    # and the un-rounded path keeps the exact value
+    _, S3, _ = O.gated_delta_ops_with_tape(q2, k2, v2, np.ones((1, 2, 1), np.float32),
+                                           np.ones((1, 2, 1), np.float32), S1)
+    np.testing.assert_array_equal(S3[0, 0, 0], [np.float32(1.0 + 3 * eps), 0.0])
+
+
 @pytest.mark.parametrize("vec", [False, True])
 def test_forward_tape_replays_to_forward_state(vec):
     """replay(tape[:n]) from S0 == state after the forward on the first n tokens."""
