@@ -239,7 +239,7 @@ int dflash_sdpa_block_causal_append(void* stream,
  * block included).  Otherwise k_new, v_new [B, Hk, M, D] are the block's rows as in the
  * append entry: read from there, stored into the pages that hold keys len..len+M-1 (which
  * the table must already map), and len_dev counts the rows already cached, block excluded.
- * No additive mask.  Returns DFLASH_NOT_SUPPORTED for a page size the kernel does not
+ * No additive mask.  Returns DFLASH_UNSUPPORTED for a page size the kernel does not
  * take.
  * ---------------------------------------------------------------------- */
 int dflash_sdpa_block_causal_paged(void* stream,

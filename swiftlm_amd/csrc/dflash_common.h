@@ -46,6 +46,13 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 int ensure_init();           // per-device one-time setup; 0 or negative hip error
 int num_compute_units();     // of the current device (cached)
 
+// Per-device setup of the kernel files, run once per device by ensure_init() under its mutex with that
+// device current: the dynamic-LDS limits of the kernels that need more than 64 KB (a function attribute is
+// per device, and setting it is not legal while a stream is being captured, so it is done here and never
+// at launch time).
+int sdpa_device_setup();
+int gdn_device_setup();
+
 // Launches one kernel.  When the thread was armed by dflash_profile_next_launch() for this kernel id,
 // the caller's events are attached to the dispatch itself (hipExtLaunchKernelGGL), so their elapsed
 // time is the kernel's own begin-to-end duration, as a profiler reports it, not a bracket around it.

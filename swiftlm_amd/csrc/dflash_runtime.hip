@@ -38,6 +38,10 @@ int ensure_init() {
         set_error("this library is built for gfx950 only; device %d is %s", dev, prop.gcnArchName);
         return DFLASH_UNSUPPORTED;
     }
+    int rc = sdpa_device_setup();
+    if (rc) return rc;
+    rc = gdn_device_setup();
+    if (rc) return rc;
     g_cus[dev] = prop.multiProcessorCount;
     g_ready[dev] = true;
     return 0;

@@ -795,23 +795,28 @@ __global__ __launch_bounds__(kThreads) void gated_delta_chunk_kernel(GdnArgs A) 
 
 template <int DK>
 static int launch_gdn_chunk(hipStream_t st, const GdnArgs& A, int B) {
-    static bool attr_done_dev[64][2];      // the attribute is per device and per instantiation
-    const size_t lds = sizeof(GdnChunkLds<DK>);
-    const int mi = A.mask ? 1 : 0;
-    int dev = 0;
-    DFLASH_HIP_TRY(hipGetDevice(&dev));
-    bool* attr_done = attr_done_dev[dev & 63];
-    if (!attr_done[mi]) {
-        if (mi) DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<true, DK>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        else DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<false, DK>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_done[mi] = true;
-    }
+    const size_t lds = sizeof(GdnChunkLds<DK>);     // the attribute that allows it is set per device by gdn_device_setup()
     dim3 grid(A.Dv / kChunkRows, B * A.Hv);
     LaunchBracket br(DFLASH_KERNEL_GDN_FORWARD, st);
     if (A.mask) br.launch(gated_delta_chunk_kernel<true, DK>, grid, dim3(kThreads), lds, A);
     else br.launch(gated_delta_chunk_kernel<false, DK>, grid, dim3(kThreads), lds, A);
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
+}
+
+template <int DK>
+static int gdn_chunk_setup() {
+    const int lds = (int)sizeof(GdnChunkLds<DK>);
+    DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<true, DK>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<false, DK>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    return DFLASH_OK;
+}
+
+int gdn_device_setup() {
+    int rc = gdn_chunk_setup<64>();
+    if (rc == DFLASH_OK) rc = gdn_chunk_setup<128>();
+    if (rc == DFLASH_OK) rc = gdn_chunk_setup<256>();
+    return rc;
 }
 
 template <typename StateT>

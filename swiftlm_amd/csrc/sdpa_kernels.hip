@@ -846,10 +846,7 @@ template <typename Tag, int D, bool MASKED, bool PAGED>
 static int launch_sdpa(hipStream_t st, const SdpaArgs& A, const CombineArgs& C, int B) {
     typedef SdpaLds<D> L;
     static_assert(L::BYTES <= 160 * 1024, "Q and the tile rings must fit the 160 KB LDS of a gfx950 CU");
-    auto kern = sdpa_partial_kernel<Tag, D, MASKED, PAGED>;
-    static const hipError_t attr_rc =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, L::BYTES);
-    DFLASH_HIP_TRY(attr_rc);
+    auto kern = sdpa_partial_kernel<Tag, D, MASKED, PAGED>;     // its dynamic-LDS limit is set per device by sdpa_device_setup()
     dim3 grid(A.S, A.Hk * A.groups_per_kv, B);
     {
         LaunchBracket br(DFLASH_KERNEL_SDPA_PARTIAL, st);
@@ -862,6 +859,23 @@ static int launch_sdpa(hipStream_t st, const SdpaArgs& A, const CombineArgs& C, 
     }
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
+}
+
+template <typename Tag, int D>
+static int sdpa_partial_setup() {
+    const int lds = SdpaLds<D>::BYTES;
+    DFLASH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(sdpa_partial_kernel<Tag, D, false, false>), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    DFLASH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(sdpa_partial_kernel<Tag, D, true, false>), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    DFLASH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(sdpa_partial_kernel<Tag, D, false, true>), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    return DFLASH_OK;
+}
+
+int sdpa_device_setup() {
+    int rc = sdpa_partial_setup<Bf16Tag, 256>();
+    if (rc == DFLASH_OK) rc = sdpa_partial_setup<Bf16Tag, 128>();
+    if (rc == DFLASH_OK) rc = sdpa_partial_setup<F16Tag, 256>();
+    if (rc == DFLASH_OK) rc = sdpa_partial_setup<F16Tag, 128>();
+    return rc;
 }
 
 }  // namespace dflash
