@@ -186,6 +186,30 @@ int dflash_sdpa_block_causal(void* stream,
                              const int32_t* kv_len_dev,
                              void* workspace, size_t workspace_bytes);
 
+/* dflash_sdpa_block_causal without a workspace argument and without any allocation.  It has no
+ * counterpart in the reference; it is for callers that cannot allocate device memory where they
+ * call it: code inside a HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * The split-KV partial rows and their statistics go to an array of
+ * DFLASH_SDPA_STATIC_SCRATCH_BYTES that lives in the library's code object (every GPU the library
+ * runs on holds its own copy until the process ends); its address is looked up once per device by
+ * dflash_init() -- call that once at set-up, outside any capture; afterwards this entry makes no
+ * allocating call (no hipMalloc / hipFree, no allocating library routine).
+ * Arguments, results and return codes are those of dflash_sdpa_block_causal; a shape whose split-KV
+ * scratch exceeds the array (about B*Hq*16 rows x splits x (2*D + 8) bytes; the benchmark shape
+ * B=1, Hq=16, Hk=2, D=256 needs 17.0 MB) returns DFLASH_UNSUPPORTED with the two sizes in
+ * dflash_last_error(), and the caller uses the workspace entry.
+ * Every call on a GPU shares that GPU's array and finds the previous call's contents in it (nothing
+ * in it has to start at zero: each call writes every statistic it later reads).  Calls that overlap
+ * on one GPU -- two streams, or two threads -- race on it; serialise them or use the workspace entry.
+ * ---------------------------------------------------------------------- */
+#define DFLASH_SDPA_STATIC_SCRATCH_BYTES (18 * 1024 * 1024)
+int dflash_sdpa_block_causal_static(void* stream,
+                                    const void* q, const void* k, const void* v,
+                                    void* out, float* lse, int dtype, float scale,
+                                    int B, int Hq, int Hk, int M, int N, int D,
+                                    int64_t kv_batch_stride, int64_t kv_head_stride,
+                                    const int32_t* kv_len_dev);
+
 /* The same attention with the reference's optional additive mask (masked partials
  * kernel, DFlashKernels.swift:546-555; selected at :783-787).  mask [B, Hq, M, N]
  * contiguous, in `dtype` (the reference casts it to the input type, :784).  A key

@@ -35,6 +35,7 @@ SIGNATURES = {
     "dflash_gdn_finish": (i32, [vp, vp, vp, vp, vp, i32, f32, i32, i32, i32, i32, i32]),
     "dflash_sdpa_workspace_bytes": (sz, [i32] * 6),
     "dflash_sdpa_block_causal": (i32, [vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp, vp, sz]),
+    "dflash_sdpa_block_causal_static": (i32, [vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp]),
     "dflash_sdpa_block_causal_masked": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp, vp, sz]),
     "dflash_sdpa_block_causal_append": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp, vp, sz]),
     "dflash_sdpa_block_causal_paged": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, i64, i64, vp, vp, vp, vp, i32, f32] + [i32] * 6 +

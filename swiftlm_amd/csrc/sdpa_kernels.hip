@@ -870,12 +870,27 @@ static int sdpa_partial_setup() {
     return DFLASH_OK;
 }
 
+// Split-KV workspace of dflash_sdpa_block_causal_static: the partial rows and their statistics live in this
+// file-scope device array instead of a caller-provided workspace, so that entry allocates nothing.  Every GPU the
+// library runs on holds its own copy, at its own address, until the process ends.  `scratch` itself is only the
+// host-side handle of the symbol: device code is handed the address that hipGetSymbolAddress returned for the
+// device at hand, never the name.
+static __device__ __align__(256) unsigned char scratch[DFLASH_SDPA_STATIC_SCRATCH_BYTES];
+static unsigned char* g_scratch_dev[64];     // per device; written once by sdpa_device_setup() under the init mutex
+
 int sdpa_device_setup() {
     int rc = sdpa_partial_setup<Bf16Tag, 256>();
     if (rc == DFLASH_OK) rc = sdpa_partial_setup<Bf16Tag, 128>();
     if (rc == DFLASH_OK) rc = sdpa_partial_setup<F16Tag, 256>();
     if (rc == DFLASH_OK) rc = sdpa_partial_setup<F16Tag, 128>();
-    return rc;
+    if (rc != DFLASH_OK) return rc;
+    int dev = 0;
+    DFLASH_HIP_TRY(hipGetDevice(&dev));
+    void* ptr = nullptr;
+    DFLASH_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    DFLASH_REQUIRE(ptr != nullptr && (uintptr_t)ptr % 256 == 0, "sdpa: the static scratch array has no usable device address");
+    g_scratch_dev[dev & 63] = static_cast<unsigned char*>(ptr);
+    return DFLASH_OK;
 }
 
 }  // namespace dflash
@@ -900,7 +915,7 @@ struct PagedKv {
 static int sdpa_common(void* stream, const void* q, const void* k, const void* v, const void* k_new, const void* v_new,
                        void* k_cache, void* v_cache, const void* mask, void* out, float* lse, int dtype, float scale, int B, int Hq, int Hk,
                        int M, int N, int D, int64_t kv_batch_stride, int64_t kv_head_stride, const int32_t* kv_len_dev,
-                       void* workspace, size_t workspace_bytes, const PagedKv* paged = nullptr) {
+                       void* workspace, size_t workspace_bytes, const PagedKv* paged = nullptr, bool static_scratch = false) {
     int rc = ensure_init();
     if (rc) return rc;
     DFLASH_REQUIRE(q && k && v && out, "sdpa: null pointer");
@@ -938,6 +953,16 @@ static int sdpa_common(void* stream, const void* q, const void* k, const void* v
     const int S = choose_splits(B, Hk, groups, N);
     size_t om, ol;
     const size_t need = ws_layout(B, Hq, S, D, &om, &ol);
+    if (static_scratch) {
+        // the library's own per-device array stands in for the workspace (address looked up at init, with that device current)
+        DFLASH_SUPPORTED(need <= (size_t)DFLASH_SDPA_STATIC_SCRATCH_BYTES,
+                         "sdpa (static): this shape needs %zu bytes of split-KV scratch, the built-in array holds %zu; "
+                         "use dflash_sdpa_block_causal with a workspace", need, (size_t)DFLASH_SDPA_STATIC_SCRATCH_BYTES);
+        int dev = 0;
+        DFLASH_HIP_TRY(hipGetDevice(&dev));
+        workspace = g_scratch_dev[dev & 63];
+        workspace_bytes = DFLASH_SDPA_STATIC_SCRATCH_BYTES;
+    }
     DFLASH_REQUIRE(workspace && workspace_bytes >= need, "sdpa: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     DFLASH_REQUIRE((uintptr_t)workspace % 256 == 0, "sdpa: workspace must be 256-byte aligned");
 
@@ -983,6 +1008,14 @@ extern "C" int dflash_sdpa_block_causal(void* stream, const void* q, const void*
                                         const int32_t* kv_len_dev, void* workspace, size_t workspace_bytes) {
     return sdpa_common(stream, q, k, v, nullptr, nullptr, nullptr, nullptr, nullptr, out, lse, dtype, scale, B, Hq, Hk, M, N, D,
                        kv_batch_stride, kv_head_stride, kv_len_dev, workspace, workspace_bytes);
+}
+
+extern "C" int dflash_sdpa_block_causal_static(void* stream, const void* q, const void* k, const void* v, void* out,
+                                               float* lse, int dtype, float scale, int B, int Hq, int Hk, int M, int N,
+                                               int D, int64_t kv_batch_stride, int64_t kv_head_stride,
+                                               const int32_t* kv_len_dev) {
+    return sdpa_common(stream, q, k, v, nullptr, nullptr, nullptr, nullptr, nullptr, out, lse, dtype, scale, B, Hq, Hk, M, N, D,
+                       kv_batch_stride, kv_head_stride, kv_len_dev, nullptr, 0, nullptr, true);
 }
 
 extern "C" int dflash_sdpa_block_causal_append(void* stream, const void* q, void* k_cache, void* v_cache,
