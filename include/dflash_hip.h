@@ -378,8 +378,15 @@ int dflash_kv_append(void* stream, void* k_cache, void* v_cache, const void* k_n
 #define DFLASH_KERNEL_TAPE_REPLAY 3
 #define DFLASH_KERNEL_GREEDY_PARTIAL 4
 #define DFLASH_KERNEL_GDN_PREPARE 5
-#define DFLASH_KERNEL_COUNT 6
+#define DFLASH_KERNEL_EMPTY 6
+#define DFLASH_KERNEL_COUNT 7
 int dflash_profile_next_launch(int kernel_id, void* start_event, void* stop_event);
+
+/* Launches a kernel that does nothing, with the given grid, block size (a multiple of 64, at most
+ * 1024) and dynamic LDS size (at most 160 KB): the cost of a launch of that shape before any work,
+ * i.e. the floor under each kernel of a verify step.  No counterpart in the reference.  Kernel id
+ * DFLASH_KERNEL_EMPTY for dflash_profile_next_launch. */
+int dflash_profile_empty_launch(void* stream, int grid_x, int grid_y, int grid_z, int threads, int lds_bytes);
 
 #ifdef __cplusplus
 }

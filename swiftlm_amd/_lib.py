@@ -18,7 +18,7 @@ F32, BF16, F16, U8 = 0, 1, 2, 3
 CACHE_TAPE, CACHE_SNAPSHOT, CACHE_MAMBA, CACHE_KV = 0, 1, 2, 3
 MAX_BATCHED_LAYERS = 64
 KERNEL_SDPA_PARTIAL, KERNEL_SDPA_COMBINE, KERNEL_GDN_FORWARD, KERNEL_TAPE_REPLAY = 0, 1, 2, 3
-KERNEL_GREEDY_PARTIAL, KERNEL_GDN_PREPARE = 4, 5
+KERNEL_GREEDY_PARTIAL, KERNEL_GDN_PREPARE, KERNEL_EMPTY = 4, 5, 6
 
 vp, i32, i64, f32, sz = C.c_void_p, C.c_int, C.c_int64, C.c_float, C.c_size_t
 vpp = C.POINTER(C.c_void_p)
@@ -50,6 +50,7 @@ SIGNATURES = {
     "dflash_rebuild_conv_state": (i32, [vp, vp, vp, vp] + [i32] * 6 + [vp]),
     "dflash_kv_append": (i32, [vp, vp, vp, vp, vp] + [i32] * 5 + [i64, i64, i32, vp, i32, vp]),
     "dflash_profile_next_launch": (i32, [i32, vp, vp]),
+    "dflash_profile_empty_launch": (i32, [vp, i32, i32, i32, i32, i32]),
     "dflash_cache_create": (vp, [i32, i32]),
     "dflash_cache_destroy": (None, [vp]),
     "dflash_cache_kind": (i32, [vp]),

@@ -22,6 +22,10 @@ void set_error(const char* fmt, ...) {
     va_end(ap);
 }
 
+// A kernel that does nothing, launched with a caller-chosen grid, block and dynamic LDS size: what a launch of
+// that shape costs on this device before any work is done (the floor under every kernel of a verify step).
+__global__ void empty_kernel() {}
+
 static std::mutex g_init_mu;
 static int g_cus[64];
 static bool g_ready[64];
@@ -38,6 +42,7 @@ int ensure_init() {
         set_error("this library is built for gfx950 only; device %d is %s", dev, prop.gcnArchName);
         return DFLASH_UNSUPPORTED;
     }
+    DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)empty_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     int rc = sdpa_device_setup();
     if (rc) return rc;
     rc = gdn_device_setup();
@@ -266,6 +271,18 @@ extern "C" int dflash_profile_next_launch(int kernel_id, void* start_event, void
     DFLASH_REQUIRE((start_event == nullptr) == (stop_event == nullptr), "profile_next_launch: pass both events or neither");
     g_bracket[kernel_id].start = (hipEvent_t)start_event;
     g_bracket[kernel_id].stop = (hipEvent_t)stop_event;
+    return DFLASH_OK;
+}
+
+extern "C" int dflash_profile_empty_launch(void* stream, int grid_x, int grid_y, int grid_z, int threads, int lds_bytes) {
+    int rc = ensure_init();
+    if (rc) return rc;
+    DFLASH_REQUIRE(grid_x >= 1 && grid_y >= 1 && grid_z >= 1 && grid_y <= 65535 && grid_z <= 65535, "empty launch: bad grid");
+    DFLASH_REQUIRE(threads >= 64 && threads <= 1024 && threads % 64 == 0, "empty launch: threads=%d is not a multiple of 64 in [64, 1024]", threads);
+    DFLASH_REQUIRE(lds_bytes >= 0 && lds_bytes <= 160 * 1024, "empty launch: lds_bytes=%d outside [0, 160 KB]", lds_bytes);
+    LaunchBracket br(DFLASH_KERNEL_EMPTY, (hipStream_t)stream);
+    br.launch(empty_kernel, dim3(grid_x, grid_y, grid_z), dim3(threads), (size_t)lds_bytes);
+    DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
 }
 

@@ -202,6 +202,39 @@ class HybridVerifyStack:
             _lib.check(rc, "tape_replay_batched")
         self.phase = 1 - ph
 
+    # -- launch shapes --------------------------------------------------------------
+    def launch_shapes(self):
+        """(grid_x, grid_y, grid_z, threads, lds_bytes) of every kernel one step launches, in launch order:
+        the shapes the library's host code picks for this configuration (csrc: launch_gdn_chunk, launch_sdpa,
+        launch_replay_nr), for pricing a step's launches with empty kernels of the same shapes.  Only the
+        benchmark's kernel choices are covered (chunked GatedDelta forward, dense or paged attention with at
+        most 8 query heads per KV head, 4 state rows per replay thread)."""
+        cfg, T = self.cfg, self.cfg.block
+        assert cfg.Dk in (64, 128, 256) and cfg.Dv % 16 == 0 and cfg.Hq // cfg.Hkv <= 8 and cfg.D in (128, 256)
+        ld = cfg.Dk + 4
+        gdn_lds = 4 * (2 * 32 * ld + 4 * 32 * 33 + 32 * 33 + 2 * 16 * 16 + 16 * 17 + 16 * 16 + 4 * 16 + 16)
+        gdn = (cfg.Dv // 16, cfg.Hv, 1, 256, gdn_lds)
+        # splits: the S whose workspace layout gives the size the library reports
+        rows = cfg.Hq * T
+        need = int(self.lib.dflash_sdpa_workspace_bytes(1, cfg.Hq, cfg.Hkv, T, self.n_max, cfg.D))
+        a256 = lambda x: (x + 255) & ~255
+        splits = [S for S in range(1, 513) if a256(a256(a256(rows * S * cfg.D * 2) + rows * S * 4) + rows * S * 4) == need]
+        assert len(splits) == 1, "cannot recover the split count from the workspace size"
+        row_bytes = cfg.D * 2
+        partial = (splits[0], cfg.Hkv, 1, 384, 4 * 32 * row_bytes + 2 * 3 * 32 * row_bytes)
+        combine = (rows, 1, 1, 256, 4 * 512 + 16 + 4 * (256 // (cfg.D // 8)) * cfg.D)
+        rpp = 256 // (cfg.Dk // 4)
+        n_gdn = len(self.gdn)
+        assert (cfg.Dv // rpp) * cfg.Hv * n_gdn >= 16 * 256 and cfg.Dv >= 4 * rpp
+        tc = 8 if cfg.Dk >= 256 else 16
+        replay = (cfg.Dv // (4 * rpp), cfg.Hv, n_gdn, 256, 4 * (tc * cfg.Dk + tc + tc * 4 * rpp + tc))
+        out = []
+        for kind in cfg.kinds():
+            out += [gdn] if kind == "gdn" else [partial, combine]
+        if n_gdn:
+            out.append(replay)
+        return out
+
     def set_acceptance(self, phase: int, commit_count: int, seed: int = 0) -> None:
         """Stage token ids for the step that will run in ``phase`` so that exactly
         ``commit_count`` tokens get committed (acceptance length commit_count - 1)."""
