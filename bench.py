@@ -310,6 +310,8 @@ def aux_kernels(lib, cfg, reps=48):
     ev.destroy()
     del sets
 
+    out["gdn_layer"] = aux_gdn_layer(lib, cfg)
+
     V = 151936
     logits = [torch.randn(T, V, generator=g, device=dev).to(bf) for _ in range(reps)]      # 48 x 4.9 MB
     mask = R.build_suppress_token_mask(V, [1, 2, 3])
@@ -328,6 +330,70 @@ def aux_kernels(lib, cfg, reps=48):
                              "shape": "T=%d V=%d bf16, uint8 suppress mask" % (T, V)}
     ev.destroy()
     return out
+
+
+def aux_gdn_layer(lib, cfg, n_layers=36, reps=30):
+    """A GatedDelta layer's body between its projections (conv + SiLU, q/k norm, gates, recurrence with tape,
+    gated norm) at the benchmark's shapes, as the three calls prepare -> forward -> finish and as the one call
+    dflash_gdn_layer (pre-ops inside the forward kernel): `n_layers` layers with their own inputs and states
+    captured into one HIP graph each way, microseconds per layer by the host clock around `reps` replays, and
+    the kernels' own durations by events on an eager pass."""
+    import torch
+    from swiftlm_amd import DFlashKernels as K, _lib
+
+    dev, bf = "cuda", torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(12)
+    B, T, Hk, Hv, Dk, Dv, Kc = 1, cfg.block, cfg.Hk, cfg.Hv, cfg.Dk, cfg.Dv, 4
+    C = 2 * Hk * Dk + Hv * Dv
+    rn = lambda *shape: torch.randn(*shape, generator=g, device=dev)
+    layers = [dict(x=rn(B, T, C).to(bf), st=rn(B, Kc - 1, C).to(bf), a=(2 * rn(B, T, Hv)).to(bf), b=rn(B, T, Hv).to(bf),
+                   w=(0.5 * rn(C, Kc)).to(bf), a_log=0.5 * rn(Hv), dt_bias=rn(Hv), s0=0.1 * rn(B, Hv, Dv, Dk),
+                   z=rn(B, T, Hv, Dv).to(bf), nw=(1 + 0.1 * rn(Dv)).to(bf)) for _ in range(n_layers)]
+    sc = dict(q_scale=1.0 / Dk, k_scale=Dk ** -0.5)
+
+    def three(l):
+        q, k, v, gg, beta, conv = K.gdn_prepare(l["x"], l["st"], l["w"], l["a"], l["b"], l["a_log"], l["dt_bias"], Hk, Hv, Dk, Dv, **sc)
+        y, s1, tape = K.gated_delta_kernel_with_tape(q, k, v, gg, beta, l["s0"])
+        return K.gdn_finish(y, l["z"], l["nw"], 1e-6, "silu"), s1, tape, k, gg, conv
+
+    def one(l):
+        r = K.gdn_layer(l["x"], l["st"], l["w"], l["a"], l["b"], l["a_log"], l["dt_bias"], l["s0"], Hk, Hv, Dk, Dv, **sc,
+                        gate=l["z"], norm_weight=l["nw"], norm_eps=1e-6, gate_kind="silu")
+        return r["out"], r["state"], r["tape"], r["k"], r["g"], r["conv_state"]
+
+    res = {"shape": "B=1 T=%d Hk=%d Hv=%d Dk=%d Dv=%d K=%d bf16, fp32 state, %d layers per graph" % (T, Hk, Hv, Dk, Dv, Kc, n_layers)}
+    same = True
+    for l in layers[:3]:
+        same = same and all(torch.equal(a, b) for a, b in zip(three(l), one(l)))
+    res["one_call_equals_three_calls_bitwise"] = bool(same)
+    side = torch.cuda.Stream()
+    for name, fn, launches in (("three_calls", three, 3), ("one_call", one, 2)):
+        torch.cuda.synchronize()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            keep = [fn(l) for l in layers]
+        torch.cuda.current_stream().wait_stream(side)
+        for _ in range(5):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            graph.replay()
+        torch.cuda.synchronize()
+        res[name] = {"us_per_layer": round((time.perf_counter() - t0) / (reps * n_layers) * 1e6, 2), "launches_per_layer": launches}
+        del graph, keep
+    for kid, name, fn in ((_lib.KERNEL_GDN_PREPARE, "gdn_prepare_kernel_us", three), (_lib.KERNEL_GDN_FORWARD, "gdn_forward_kernel_us", three),
+                          (_lib.KERNEL_GDN_FINISH, "gdn_finish_kernel_us", three), (_lib.KERNEL_GDN_LAYER, "gdn_layer_kernel_us", one)):
+        ev = HipEvents()
+        for l in layers:
+            e0, e1 = ev.pair()
+            _lib.check(lib.dflash_profile_next_launch(kid, e0, e1), "profile_next_launch")
+            fn(l)
+        torch.cuda.synchronize()
+        res[name] = round(float(np.median(ev.durations_us())), 2)
+        ev.destroy()
+    return res
 
 
 def main():

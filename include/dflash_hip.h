@@ -157,6 +157,42 @@ int dflash_gdn_finish(void* stream, const void* y, const void* gate, const void*
                       int in_dtype, float norm_eps, int gate_kind, int B, int T, int Hv, int Dv);
 
 /* ------------------------------------------------------------------------
+ * One GatedDelta layer of the verify block, from its projections to the gated norm, in one call:
+ * the body of the layer between its input and output projections
+ * (Sources/SwiftLM/KimiLinearDFlash.swift:351-378: short conv + SiLU, q/k normalisation, gates,
+ * the recurrence through DFlashKernelProvider.gatedDeltaKernelWithTape, oNorm(out) * act(gate)).
+ * Equivalent to dflash_gdn_prepare -> dflash_gated_delta_tape -> dflash_gdn_finish, bit for bit,
+ * in two launches instead of three: the pre-ops run inside the forward kernel's load phase, so
+ * q, k, v, g and beta never travel through memory; the gated norm stays a launch of its own
+ * because it normalises over the Dv rows of a head, which the forward spreads over several
+ * workgroups.
+ *   inputs    mixed_qkv, conv_state_in (or NULL), conv_weight, a_logits [B,T,Hv], b_logits,
+ *             A_log, dt_bias [Hv], q_scale, k_scale, norm_eps as for dflash_gdn_prepare;
+ *             state_in [B,Hv,Dv,Dk] float32
+ *   outputs   state_out (float32), tape_out [B,T,Hv,Dv] float32, y_out [B,T,Hv,Dv] (the
+ *             recurrence's read-out before the norm), conv_state_out [B,K-1,C];
+ *             k_out [B,T,Hk,Dk] and g_out [B,T,Hv]: what recordTape keeps for the replay
+ *             (RecurrentRollbackCache.swift:75-85), NULL to skip;
+ *             q_out, v_out, beta_out: optional copies of the other pre-op results, NULL to skip
+ *   gate      NULL: stop after the recurrence.  Otherwise gate [B,T,Hv,Dv], out_norm_weight [Dv],
+ *             out_norm_eps, gate_kind and out [B,T,Hv,Dv] as for dflash_gdn_finish.
+ * Covers the verify block: float32 state, one decay per head and step, no step mask, K == 4,
+ * T <= 16, Dk in {64, 128, 256}, Dv a multiple of 16.  Anything else returns
+ * DFLASH_UNSUPPORTED and the caller issues the three calls.
+ * ---------------------------------------------------------------------- */
+int dflash_gdn_layer(void* stream,
+                     const void* mixed_qkv, const void* conv_state_in, const void* conv_weight,
+                     const void* a_logits, const void* b_logits,
+                     const float* A_log, const float* dt_bias, int in_dtype,
+                     float q_scale, float k_scale, float norm_eps,
+                     const void* state_in, void* state_out,
+                     void* k_out, void* g_out, float* tape_out, void* conv_state_out, void* y_out,
+                     const void* gate, const void* out_norm_weight, float out_norm_eps, int gate_kind,
+                     void* out,
+                     void* q_out, void* v_out, void* beta_out,
+                     int B, int T, int Hk, int Hv, int Dk, int Dv, int K);
+
+/* ------------------------------------------------------------------------
  * Block-causal batched GQA SDPA for the verify block.  Replaces
  * DFlashKernels.batchedSDPA2Pass (DFlashKernels.swift:737-815; Metal partials
  * :563-649, reduce :661-720); unlike it, covers every shape sdpaFallback
@@ -379,7 +415,9 @@ int dflash_kv_append(void* stream, void* k_cache, void* v_cache, const void* k_n
 #define DFLASH_KERNEL_GREEDY_PARTIAL 4
 #define DFLASH_KERNEL_GDN_PREPARE 5
 #define DFLASH_KERNEL_EMPTY 6
-#define DFLASH_KERNEL_COUNT 7
+#define DFLASH_KERNEL_GDN_LAYER 7
+#define DFLASH_KERNEL_GDN_FINISH 8
+#define DFLASH_KERNEL_COUNT 9
 int dflash_profile_next_launch(int kernel_id, void* start_event, void* stop_event);
 
 /* Launches a kernel that does nothing, with the given grid, block size (a multiple of 64, at most

@@ -18,7 +18,7 @@ F32, BF16, F16, U8 = 0, 1, 2, 3
 CACHE_TAPE, CACHE_SNAPSHOT, CACHE_MAMBA, CACHE_KV = 0, 1, 2, 3
 MAX_BATCHED_LAYERS = 64
 KERNEL_SDPA_PARTIAL, KERNEL_SDPA_COMBINE, KERNEL_GDN_FORWARD, KERNEL_TAPE_REPLAY = 0, 1, 2, 3
-KERNEL_GREEDY_PARTIAL, KERNEL_GDN_PREPARE, KERNEL_EMPTY = 4, 5, 6
+KERNEL_GREEDY_PARTIAL, KERNEL_GDN_PREPARE, KERNEL_EMPTY, KERNEL_GDN_LAYER, KERNEL_GDN_FINISH = 4, 5, 6, 7, 8
 
 vp, i32, i64, f32, sz = C.c_void_p, C.c_int, C.c_int64, C.c_float, C.c_size_t
 vpp = C.POINTER(C.c_void_p)
@@ -33,6 +33,7 @@ SIGNATURES = {
     "dflash_gated_delta_tape": (i32, [vp, vp, vp, vp, vp, i32, vp, i32, vp, vp, i32, vp, vp, vp, i32] + [i32] * 6),
     "dflash_gdn_prepare": (i32, [vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, f32, f32, f32, vp, vp, vp, vp, vp, vp] + [i32] * 7),
     "dflash_gdn_finish": (i32, [vp, vp, vp, vp, vp, i32, f32, i32, i32, i32, i32, i32]),
+    "dflash_gdn_layer": (i32, [vp] * 8 + [i32, f32, f32, f32] + [vp] * 9 + [f32, i32] + [vp] * 4 + [i32] * 7),
     "dflash_sdpa_workspace_bytes": (sz, [i32] * 6),
     "dflash_sdpa_block_causal": (i32, [vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp, vp, sz]),
     "dflash_sdpa_block_causal_static": (i32, [vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp]),

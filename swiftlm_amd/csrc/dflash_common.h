@@ -88,12 +88,9 @@ __device__ __forceinline__ float to_float(float x) { return x; }
 __device__ __forceinline__ float to_float(bf16_t x) { return __uint_as_float(((uint32_t)x.bits) << 16); }
 __device__ __forceinline__ float to_float(f16_t x) { return (float)x.v; }
 
-// round-to-nearest-even, NaN preserved
+// round-to-nearest-even, NaN stays NaN: the hardware convert of gfx950 (v_cvt_pk_bf16_f32)
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
 }
 
 template <typename T> __device__ __forceinline__ T from_float(float f);
@@ -124,6 +121,28 @@ __device__ __forceinline__ void store4(bf16_t* p, float4 v) {
 }
 __device__ __forceinline__ void store4(f16_t* p, float4 v) {
     p[0].v = (_Float16)v.x; p[1].v = (_Float16)v.y; p[2].v = (_Float16)v.z; p[3].v = (_Float16)v.w;
+}
+
+// ---- GatedDelta layer formulas shared by the pre-op kernel and the one-launch layer kernel ----
+// Both kernels must round identically, so the expressions live here once.
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(__expf(z)); }
+// 1 / (1 + e^-z) with the hardware exponential and reciprocal (about 2 ulp)
+__device__ __forceinline__ float sigmoid_f(float z) { return __builtin_amdgcn_rcpf(1.f + __expf(-z)); }
+// The product is pinned as a float so that a following narrowing convert cannot be merged with the multiply
+// (a merged multiply-convert rounds once, the two-step form twice: kernels that must agree bit for bit would not).
+__device__ __forceinline__ float silu_f(float y) {
+    float r = y * sigmoid_f(y);
+    asm("" : "+v"(r));
+    return r;
+}
+// g = exp(-exp(A_log) * softplus(a + dt_bias)) (Sources/SwiftLM/KimiLinearDFlash.swift:390)
+__device__ __forceinline__ float gdn_decay(float a_logit, float dt_bias, float a_log) {
+    const float z = a_logit + dt_bias;
+    return __expf(-__expf(a_log) * softplus_f(z));
+}
+// scale * rsqrt(mean(x^2) + eps) for a head of `dim` channels whose squares sum to `sumsq` (:362-363)
+__device__ __forceinline__ float gdn_norm_scale(float sumsq, int dim, float eps, float scale) {
+    return scale * rsqrtf(sumsq / (float)dim + eps);
 }
 
 // mask element of run-time type -> "this step runs"
@@ -169,6 +188,24 @@ template <int LANES> __device__ __forceinline__ float group_sum(float x) {
     x = dpp_add<0x4E>(x);                          // quad_perm [2,3,0,1]
     if (LANES >= 8) x = dpp_add<0x141>(x);         // row_half_mirror
     if (LANES >= 16) x = dpp_add<0x140>(x);        // row_mirror
+    return x;
+}
+
+// Sum over groups of LANES (a power of two, 4..64) consecutive lanes as a butterfly: neighbours first (lane bit 0),
+// then bit 1, and so on; every lane of the group receives the total.  Floating-point addition is commutative, so
+// every lane holds the same bits, and two kernels that both use this order agree bit for bit.  Bits 0-3 stay inside
+// a 16-lane DPP row; bit 4 and bit 5 use gfx950's v_permlane16_swap / v_permlane32_swap.
+template <int LANES> __device__ __forceinline__ float butterfly_sum(float x) {
+    static_assert(LANES == 4 || LANES == 8 || LANES == 16 || LANES == 32 || LANES == 64, "group size");
+    x = group_sum<(LANES > 16 ? 16 : LANES)>(x);
+    if (LANES >= 32) {
+        auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+        x = __fadd_rn(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    }
+    if (LANES >= 64) {
+        auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+        x = __fadd_rn(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    }
     return x;
 }
 

@@ -364,6 +364,23 @@ struct GdnArgs {
     int T, Hk, Hv, Dv;
 };
 
+// Inputs of the layer's pre-ops when they run inside the forward kernel (gdn_layer_kernel): the short
+// conv + SiLU over q|k|v, the q/k normalisation and the gate formulas of dflash_gdn_prepare.
+struct GdnPrep {
+    const void* x;            // mixed_qkv [B,T,C]
+    const void* conv_in;      // [B,K-1,C] or null (zeros)
+    const void* weight;       // [C,K]
+    const void* a;            // [B,T,Hv]
+    const void* b;            // [B,T,Hv]
+    const float* a_log;       // [Hv]
+    const float* dt_bias;     // [Hv]
+    void *q_out, *k_out, *v_out, *g_out, *beta_out;   // each may be null
+    void* conv_out;           // [B,K-1,C]
+    float q_scale, k_scale, eps;
+    int C;
+};
+constexpr int kLayerTaps = 4;  // conv kernel size the one-launch layer kernel is built for
+
 constexpr int kGdnChunk = 16;  // steps staged in LDS at a time
 
 // LPR lanes share one state row; each keeps DK/LPR channels as float4 pieces
@@ -584,11 +601,20 @@ template <int S> struct SolveStep {
     }
 };
 
-template <bool HAS_MASK, int DK>
-__global__ __launch_bounds__(kThreads) void gated_delta_chunk_kernel(GdnArgs A) {
+template <bool HAS_MASK, int DK, bool FUSED>
+__device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& P) {
     using Lds = GdnChunkLds<DK>;
     extern __shared__ __align__(16) unsigned char gdn_chunk_smem[];
     Lds& L = *reinterpret_cast<Lds*>(gdn_chunk_smem);
+    // Every kernel argument is asked for here, in one burst of scalar loads.  Left alone the compiler fetches
+    // them where they are first used, in three or four dependent rounds, and each round that touches a new
+    // cache line of the argument block is a trip to memory on the way to the first global load.
+    asm volatile("" ::"s"(A.q), "s"(A.k), "s"(A.v), "s"(A.g), "s"(A.beta), "s"(A.mask), "s"(A.state_in), "s"(A.state_out),
+                 "s"(A.y), "s"(A.tape), "s"(A.in_dtype), "s"(A.mask_dtype), "s"(A.T), "s"(A.Hk), "s"(A.Hv), "s"(A.Dv));
+    if constexpr (FUSED)
+        asm volatile("" ::"s"(P.x), "s"(P.conv_in), "s"(P.weight), "s"(P.a), "s"(P.b), "s"(P.a_log), "s"(P.dt_bias),
+                     "s"(P.q_out), "s"(P.k_out), "s"(P.v_out), "s"(P.g_out), "s"(P.beta_out), "s"(P.conv_out),
+                     "s"(P.q_scale), "s"(P.k_scale), "s"(P.eps), "s"(P.C));
     constexpr int E = DK / 64;             // channels per lane in the state-update product (16 lanes x E x 4 waves = DK)
     static_assert(DK % 64 == 0, "chunked gated delta needs Dk to be a multiple of 64");
 
@@ -612,7 +638,16 @@ __global__ __launch_bounds__(kThreads) void gated_delta_chunk_kernel(GdnArgs A) 
         return;
     }
 
-    // Stage one chunk: every global load of the chunk (and of the state tile, first chunk only) is issued
+    // The state tile is the coldest and largest operand: its loads go out first, ahead of the index arithmetic of
+    // everything else.
+    float4 sv0[NV];
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int i = tid + u * kThreads, r = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
+        sv0[u] = load4(s_in + (size_t)r * DK + c4);
+    }
+
+    // Stage one chunk: every global load of the chunk (the state tile is already on its way) is issued
     // before the first conversion or LDS store, so the chunk pays one memory round trip, not one per array.
     // Steps >= tc are identity steps.  Elem is the element type of q/k/v/g/beta.
     auto stage = [&](auto elem_tag, int t0, int tc, bool with_state) {
@@ -622,15 +657,8 @@ __global__ __launch_bounds__(kThreads) void gated_delta_chunk_kernel(GdnArgs A) 
         const Elem* vp = reinterpret_cast<const Elem*>(A.v);
         const Elem* gp = reinterpret_cast<const Elem*>(A.g);
         const Elem* bp = reinterpret_cast<const Elem*>(A.beta);
-        float4 sv[NV], kv[NV], qv[NV];
+        float4 kv[NV], qv[NV];
         const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (with_state) {
-#pragma unroll
-            for (int u = 0; u < NV; ++u) {
-                const int i = tid + u * kThreads, r = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
-                sv[u] = load4(s_in + (size_t)r * DK + c4);
-            }
-        }
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
             const int i = tid + u * kThreads, t = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
@@ -655,7 +683,7 @@ __global__ __launch_bounds__(kThreads) void gated_delta_chunk_kernel(GdnArgs A) 
 #pragma unroll
             for (int u = 0; u < NV; ++u) {
                 const int i = tid + u * kThreads, r = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
-                store4(&L.x[r][c4], sv[u]);
+                store4(&L.x[r][c4], sv0[u]);
             }
         }
 #pragma unroll
@@ -674,12 +702,164 @@ __global__ __launch_bounds__(kThreads) void gated_delta_chunk_kernel(GdnArgs A) 
         }
     };
 
-    for (int t0 = 0; t0 < A.T; t0 += kChunkSteps) {
+    // The same with the layer's pre-ops done on the way in (one chunk, T <= 16, kLayerTaps conv taps): instead of
+    // q, k, v, g, beta the workgroup reads the raw projections -- for every (step, 4 channels) of its key head the
+    // K window rows of q and of k, for its 16 value rows K single elements per step -- and the conv taps, all in one
+    // round trip with the state tile; conv -> SiLU -> per-head RMS scale (sum of squares over the DK/4 lanes that
+    // share a step) -> rounded to the element type exactly as dflash_gdn_prepare stores them, so that the recurrence
+    // sees bit-identical operands.  What the rollback cache records (k, g, the conv window) and the optional q, v,
+    // beta are written by the first row tile of a head (q, k: of the first value head of the key head's group).
+    auto stage_fused = [&](auto elem_tag, int tc) {
+        using Elem = decltype(elem_tag);
+        constexpr int KT = kLayerTaps, keep = KT - 1, LPT = DK / 4;
+        const int C = P.C;
+        const Elem* x = reinterpret_cast<const Elem*>(P.x) + (size_t)b * A.T * C;
+        const Elem* cs = P.conv_in ? reinterpret_cast<const Elem*>(P.conv_in) + (size_t)b * keep * C : nullptr;
+        const Elem* wt = reinterpret_cast<const Elem*>(P.weight);
+        const int cq = hk * DK, ck = (A.Hk + hk) * DK, cv = 2 * A.Hk * DK + hv * A.Dv + row0;
+        const int c4 = (tid % LPT) * 4;
+        // Window row r of the concatenation [conv_in (keep rows) ; x (T rows)]; without conv_in its rows are zeros
+        // (a valid address is read and the value dropped).  Selects, no branches: a branch around a load makes the
+        // compiler wait for that load before it issues the next one.
+        const Elem* csz = cs ? cs : x;
+        auto win_row = [&](int r) -> const Elem* {
+            const bool in_x = r >= keep;
+            const int rr = in_x ? r - keep : (cs ? r : 0);
+            return (in_x ? x : csz) + (size_t)rr * C;
+        };
+        float4 kw[NV][KT], qw[NV][KT], ktap[4], qtap[4], vtap;
+        float vw[KT];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {               // [m] = the KT taps of channel c4 + m
+            ktap[m] = load4(wt + (size_t)(ck + c4 + m) * KT);
+            qtap[m] = load4(wt + (size_t)(cq + c4 + m) * KT);
+        }
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int t = (tid + u * kThreads) / LPT, tl = t < tc ? t : tc - 1;
+#pragma unroll
+            for (int j = 0; j < KT; ++j) {
+                const Elem* src = win_row(tl + j);
+                kw[u][j] = load4(src + ck + c4);
+                qw[u][j] = load4(src + cq + c4);
+            }
+        }
+        const int tvl = ts < tc ? ts : tc - 1;
+#pragma unroll
+        for (int j = 0; j < KT; ++j) vw[j] = to_float(win_row(tvl + j)[cv + tt]);
+        vtap = load4(wt + (size_t)(cv + tt) * KT);
+        // gate inputs: every thread reads them (step tid mod 16), so that no load sits inside a branch
+        const int tg = (tid % kChunkSteps) < tc ? (tid % kChunkSteps) : tc - 1;
+        const size_t btg = ((size_t)b * A.T + tg) * A.Hv + hv;
+        const float av = to_float(reinterpret_cast<const Elem*>(P.a)[btg]);
+        const float bv = to_float(reinterpret_cast<const Elem*>(P.b)[btg]);
+        const float alog = P.a_log[hv];
+        const float dtb = P.dt_bias[hv];
+        // ---- every load is out; now the arithmetic ----
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int i = tid + u * kThreads, r = i / (DK / 4), cc = (i % (DK / 4)) * 4;
+            store4(&L.x[r][cc], sv0[u]);
+        }
+        const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        const bool first_tile = blockIdx.x == 0;
+        const bool qk_owner = first_tile && (hv % (A.Hv / A.Hk)) == 0;
+        auto conv4 = [&](const float4 (&w)[KT], const float4 (&tap)[4], int tl) -> float4 {
+            float o[4];
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const float tp[4] = {tap[m].x, tap[m].y, tap[m].z, tap[m].w};
+                float acc = 0.f;
+#pragma unroll
+                for (int j = 0; j < KT; ++j) {
+                    const float wj[4] = {w[j].x, w[j].y, w[j].z, w[j].w};
+                    const float win = (tl + j < keep && !cs) ? 0.f : wj[m];
+                    acc = fmaf(win, tp[j], acc);
+                }
+                o[m] = silu_f(acc);
+            }
+            return make_float4(o[0], o[1], o[2], o[3]);
+        };
+        auto head_scale = [&](float4 y, float sc) -> float {
+            float ss = __fadd_rn(__fadd_rn(__fmul_rn(y.x, y.x), __fmul_rn(y.y, y.y)),
+                                 __fadd_rn(__fmul_rn(y.z, y.z), __fmul_rn(y.w, y.w)));
+            return gdn_norm_scale(butterfly_sum<LPT>(ss), DK, P.eps, sc);
+        };
+        auto round4 = [](float4 y, float sc) -> float4 {
+            return make_float4(requant<Elem>(y.x * sc), requant<Elem>(y.y * sc), requant<Elem>(y.z * sc), requant<Elem>(y.w * sc));
+        };
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int t = (tid + u * kThreads) / LPT, tl = t < tc ? t : tc - 1;
+            const float4 kc = conv4(kw[u], ktap, tl), qc = conv4(qw[u], qtap, tl);
+            const float4 k4 = round4(kc, head_scale(kc, P.k_scale)), q4 = round4(qc, head_scale(qc, P.q_scale));
+            const bool live = t < tc;
+            store4(&L.x[16 + t][c4], live ? k4 : zero4);
+            store4(&L.y[t][c4], live ? k4 : zero4);
+            store4(&L.y[16 + t][c4], live ? q4 : zero4);
+            if (qk_owner && live) {
+                const size_t o = (((size_t)b * A.T + t) * A.Hk + hk) * DK + c4;
+                if (P.k_out) store4(reinterpret_cast<Elem*>(P.k_out) + o, k4);
+                if (P.q_out) store4(reinterpret_cast<Elem*>(P.q_out) + o, q4);
+                if (t == tc - 1) {                  // the new conv window: rows 1..K-1 of the last step's window
+                    Elem* dst = reinterpret_cast<Elem*>(P.conv_out) + (size_t)b * keep * C;
+#pragma unroll
+                    for (int j = 1; j < KT; ++j) {
+                        const bool z = (tl + j < keep && !cs);
+                        store4(dst + (size_t)(j - 1) * C + ck + c4, z ? zero4 : kw[u][j]);
+                        store4(dst + (size_t)(j - 1) * C + cq + c4, z ? zero4 : qw[u][j]);
+                    }
+                }
+            }
+        }
+        {
+            const float tp[4] = {vtap.x, vtap.y, vtap.z, vtap.w};
+            float acc = 0.f;
+#pragma unroll
+            for (int j = 0; j < KT; ++j) acc = fmaf((tvl + j < keep && !cs) ? 0.f : vw[j], tp[j], acc);
+            const float vv = requant<Elem>(silu_f(acc));
+            L.v[ts][tt] = ts < tc ? vv : 0.f;
+            if (ts < tc) {
+                if (P.v_out)
+                    reinterpret_cast<Elem*>(P.v_out)[(((size_t)b * A.T + ts) * A.Hv + hv) * A.Dv + row0 + tt] = from_float<Elem>(vv);
+                if (ts == tc - 1) {
+                    Elem* dst = reinterpret_cast<Elem*>(P.conv_out) + (size_t)b * keep * C + cv + tt;
+#pragma unroll
+                    for (int j = 1; j < KT; ++j)
+                        dst[(size_t)(j - 1) * C] = from_float<Elem>((tvl + j < keep && !cs) ? 0.f : vw[j]);
+                }
+            }
+        }
+        if (tid < kChunkSteps) {
+            const bool on = tid < tc;
+            const float gv = requant<Elem>(gdn_decay(av, dtb, alog));
+            const float be = requant<Elem>(sigmoid_f(bv));
+            L.on[tid] = on;
+            L.g[tid] = on ? gv : 1.f;
+            L.beta[tid] = on ? be : 0.f;
+            if (first_tile && on) {
+                const size_t o = ((size_t)b * A.T + tid) * A.Hv + hv;
+                if (P.g_out) reinterpret_cast<Elem*>(P.g_out)[o] = from_float<Elem>(gv);
+                if (P.beta_out) reinterpret_cast<Elem*>(P.beta_out)[o] = from_float<Elem>(be);
+            }
+        }
+    };
+
+    // One chunk of up to 16 steps.  The first chunk (the only one of a verify block) is straight-line code ahead of
+    // the loop over the rest: inside the loop the compiler hoists every invariant of the whole body above the first
+    // load and carries waits round the back edge.
+    auto run_chunk = [&](const int t0) {
         const int tc = (A.T - t0) < kChunkSteps ? (A.T - t0) : kChunkSteps;
         const bool last_chunk = t0 + kChunkSteps >= A.T;
-        if (A.in_dtype == DFLASH_BF16) stage(bf16_t{}, t0, tc, t0 == 0);
-        else if (A.in_dtype == DFLASH_F16) stage(f16_t{}, t0, tc, t0 == 0);
-        else stage(float{}, t0, tc, t0 == 0);
+        if constexpr (FUSED) {
+            if (A.in_dtype == DFLASH_BF16) stage_fused(bf16_t{}, tc);
+            else if (A.in_dtype == DFLASH_F16) stage_fused(f16_t{}, tc);
+            else stage_fused(float{}, tc);
+        } else {
+            if (A.in_dtype == DFLASH_BF16) stage(bf16_t{}, t0, tc, t0 == 0);
+            else if (A.in_dtype == DFLASH_F16) stage(f16_t{}, t0, tc, t0 == 0);
+            else stage(float{}, t0, tc, t0 == 0);
+        }
         __syncthreads();
 
         // ---- [S_0 ; k] x [k | q]^T, wave w contracting channels w*DK/4 .. +DK/4-1 ----
@@ -783,14 +963,43 @@ __global__ __launch_bounds__(kThreads) void gated_delta_chunk_kernel(GdnArgs A) 
                     for (int e = 0; e < E; ++e) s_out[(size_t)(4 * kk + v) * DK + base + e] = cacc[e][v];
             } else {
                 __syncthreads();           // every wave has read the old tile
+                // One row at a time, with a compiler barrier between the rows: when the stores of rows 2 and 3 are
+                // paired into one two-address LDS store (possible at DK = 64, where both offsets fit its 8-bit
+                // fields) this compiler has emitted a wrong first offset.
 #pragma unroll
-                for (int v = 0; v < 4; ++v)
+                for (int v = 0; v < 4; ++v) {
 #pragma unroll
                     for (int e = 0; e < E; ++e) L.x[4 * kk + v][base + e] = cacc[e][v];
+                    asm volatile("" ::: "memory");
+                }
                 // the staging barrier of the next chunk orders these writes before their readers
             }
         }
-    }
+    };
+    run_chunk(0);
+    if constexpr (!FUSED)
+        for (int t0 = kChunkSteps; t0 < A.T; t0 += kChunkSteps) run_chunk(t0);
+}
+
+template <bool HAS_MASK, int DK>
+__global__ __launch_bounds__(kThreads) void gated_delta_chunk_kernel(GdnArgs A) {
+    gdn_chunk_body<HAS_MASK, DK, false>(A, GdnPrep{});
+}
+
+// One GatedDelta layer from its projections to the recurrence's outputs in one launch.
+template <int DK>
+__global__ __launch_bounds__(kThreads) void gdn_layer_kernel(GdnArgs A, GdnPrep P) {
+    gdn_chunk_body<false, DK, true>(A, P);
+}
+
+template <int DK>
+static int launch_gdn_layer(hipStream_t st, const GdnArgs& A, const GdnPrep& P, int B) {
+    const size_t lds = sizeof(GdnChunkLds<DK>);
+    dim3 grid(A.Dv / kChunkRows, B * A.Hv);
+    LaunchBracket br(DFLASH_KERNEL_GDN_LAYER, st);
+    br.launch(gdn_layer_kernel<DK>, grid, dim3(kThreads), lds, A, P);
+    DFLASH_HIP_TRY(hipGetLastError());
+    return DFLASH_OK;
 }
 
 template <int DK>
@@ -809,6 +1018,7 @@ static int gdn_chunk_setup() {
     const int lds = (int)sizeof(GdnChunkLds<DK>);
     DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<true, DK>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<false, DK>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gdn_layer_kernel<DK>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     return DFLASH_OK;
 }
 
@@ -923,4 +1133,44 @@ extern "C" int dflash_gated_delta_tape(void* stream, const void* q, const void* 
         case DFLASH_BF16: return launch_gdn_state<bf16_t>((hipStream_t)stream, A, B, g_ndim, Dk);
         default: return launch_gdn_state<f16_t>((hipStream_t)stream, A, B, g_ndim, Dk);
     }
+}
+
+extern "C" int dflash_gdn_layer(void* stream, const void* mixed_qkv, const void* conv_state_in, const void* conv_weight,
+                                const void* a_logits, const void* b_logits, const float* a_log, const float* dt_bias,
+                                int in_dtype, float q_scale, float k_scale, float norm_eps, const void* state_in,
+                                void* state_out, void* k_out, void* g_out, float* tape_out, void* conv_state_out,
+                                void* y_out, const void* gate, const void* out_norm_weight, float out_norm_eps,
+                                int gate_kind, void* out, void* q_out, void* v_out, void* beta_out, int B, int T, int Hk,
+                                int Hv, int Dk, int Dv, int K) {
+    int rc = ensure_init();
+    if (rc) return rc;
+    DFLASH_REQUIRE(B > 0 && T > 0 && Hk > 0 && Hv > 0 && Dk > 0 && Dv > 0, "gdn_layer: non-positive dimension");
+    DFLASH_REQUIRE(Hv % Hk == 0, "gdn_layer: Hv=%d is not a multiple of Hk=%d", Hv, Hk);
+    DFLASH_REQUIRE(mixed_qkv && conv_weight && a_logits && b_logits && a_log && dt_bias, "gdn_layer: null input");
+    DFLASH_REQUIRE(state_in && state_out && tape_out && y_out && conv_state_out, "gdn_layer: null output");
+    DFLASH_REQUIRE(state_in != state_out, "gdn_layer: state_in aliases state_out");
+    DFLASH_REQUIRE(conv_state_out != conv_state_in, "gdn_layer: conv_state_out aliases conv_state_in");
+    DFLASH_REQUIRE(!gate || (out_norm_weight && out), "gdn_layer: a gate needs out_norm_weight and out");
+    DFLASH_REQUIRE(gate_kind == 0 || gate_kind == 1, "gdn_layer: gate_kind must be 0 (sigmoid) or 1 (silu)");
+    DFLASH_REQUIRE((long)B * Hv <= 65535, "gdn_layer: B*Hv too large for one launch");
+    DFLASH_SUPPORTED(in_dtype == DFLASH_F32 || in_dtype == DFLASH_BF16 || in_dtype == DFLASH_F16, "gdn_layer: bad in_dtype %d", in_dtype);
+    DFLASH_SUPPORTED(K == kLayerTaps, "gdn_layer: conv kernel size %d (the one-launch layer is built for %d)", K, kLayerTaps);
+    DFLASH_SUPPORTED(T <= kChunkSteps, "gdn_layer: T=%d above one chunk of %d steps", T, kChunkSteps);
+    DFLASH_SUPPORTED(Dv % kChunkRows == 0 && (Dk == 64 || Dk == 128 || Dk == 256), "gdn_layer: Dk=%d / Dv=%d outside the chunked kernel", Dk, Dv);
+
+    GdnArgs A;
+    A.q = A.k = A.v = A.g = A.beta = A.mask = nullptr;
+    A.state_in = state_in; A.state_out = state_out; A.y = y_out; A.tape = tape_out;
+    A.in_dtype = in_dtype; A.mask_dtype = 0; A.T = T; A.Hk = Hk; A.Hv = Hv; A.Dv = Dv;
+    GdnPrep P;
+    P.x = mixed_qkv; P.conv_in = conv_state_in; P.weight = conv_weight; P.a = a_logits; P.b = b_logits;
+    P.a_log = a_log; P.dt_bias = dt_bias; P.q_out = q_out; P.k_out = k_out; P.v_out = v_out; P.g_out = g_out;
+    P.beta_out = beta_out; P.conv_out = conv_state_out; P.q_scale = q_scale; P.k_scale = k_scale; P.eps = norm_eps;
+    P.C = 2 * Hk * Dk + Hv * Dv;
+    hipStream_t st = (hipStream_t)stream;
+    if (Dk == 64) rc = launch_gdn_layer<64>(st, A, P, B);
+    else if (Dk == 128) rc = launch_gdn_layer<128>(st, A, P, B);
+    else rc = launch_gdn_layer<256>(st, A, P, B);
+    if (rc || !gate) return rc;
+    return dflash_gdn_finish(stream, y_out, gate, out_norm_weight, out, in_dtype, out_norm_eps, gate_kind, B, T, Hv, Dv);
 }

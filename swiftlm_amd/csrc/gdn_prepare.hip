@@ -31,9 +31,6 @@ struct PrepareArgs {
 
 constexpr int kPrepMaxTaps = 8;
 
-__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(__expf(z)); }
-__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + __expf(-z)); }
-
 // Grid: x = head block (Hk q heads, Hk k heads, Hv v heads, then gate blocks), y = t, z = b.
 // Block: max(Dk, Dv) threads rounded up to a multiple of 64.
 template <typename Elem>
@@ -49,8 +46,8 @@ __global__ void gdn_prepare_kernel(PrepareArgs A) {
             const int h = hb - n_conv;                       // one block per value head, one thread per channel
             if (tid < A.Dk) {
                 const size_t o = (bt * A.Hv + h) * A.Dk + tid;
-                const float z = to_float(reinterpret_cast<const Elem*>(A.a)[o]) + A.dt_bias[h * A.Dk + tid];
-                reinterpret_cast<Elem*>(A.g)[o] = from_float<Elem>(__expf(-__expf(A.a_log[h]) * softplus_f(z)));
+                reinterpret_cast<Elem*>(A.g)[o] = from_float<Elem>(
+                    gdn_decay(to_float(reinterpret_cast<const Elem*>(A.a)[o]), A.dt_bias[h * A.Dk + tid], A.a_log[h]));
             }
             if (tid == 0) {
                 const size_t o = bt * A.Hv + h;
@@ -59,8 +56,8 @@ __global__ void gdn_prepare_kernel(PrepareArgs A) {
         } else {
             for (int h = tid; h < A.Hv; h += blockDim.x) {   // a single block
                 const size_t o = bt * A.Hv + h;
-                const float z = to_float(reinterpret_cast<const Elem*>(A.a)[o]) + A.dt_bias[h];
-                reinterpret_cast<Elem*>(A.g)[o] = from_float<Elem>(__expf(-__expf(A.a_log[h]) * softplus_f(z)));
+                reinterpret_cast<Elem*>(A.g)[o] = from_float<Elem>(
+                    gdn_decay(to_float(reinterpret_cast<const Elem*>(A.a)[o]), A.dt_bias[h], A.a_log[h]));
                 reinterpret_cast<Elem*>(A.beta)[o] = from_float<Elem>(sigmoid_f(to_float(reinterpret_cast<const Elem*>(A.b)[o])));
             }
         }
@@ -95,7 +92,7 @@ __global__ void gdn_prepare_kernel(PrepareArgs A) {
     float y = 0.f;
 #pragma unroll
     for (int j = 0; j < kPrepMaxTaps; ++j) y = fmaf(win[j], tap[j], y);
-    y = y * sigmoid_f(y);                                            // silu (:291)
+    y = silu_f(y);                                                   // silu (:291)
 
     // the new conv window: the last K-1 rows of the concatenation (:292), i.e. rows 1..K-1 of the
     // window of the last step
@@ -111,13 +108,19 @@ __global__ void gdn_prepare_kernel(PrepareArgs A) {
         return;
     }
     // ---- q, k: scale * x * rsqrt(mean(x^2) + eps) over the head (:362-363) ----
-    float ss = on ? y * y : 0.f;
-    for (int o = 32; o >= 1; o >>= 1) ss += __shfl_xor(ss, o);
+    // The squares are summed pairwise, neighbours first (channel bit 0, then bit 1, ...), which is the order
+    // the one-launch layer kernel reproduces with four channels per lane: both give the same bits.
+    float ss = butterfly_sum<64>(on ? __fmul_rn(y, y) : 0.f);
     if ((tid & 63) == 0) red_s[tid >> 6] = ss;
     __syncthreads();
-    float tot = 0.f;
-    for (int i = 0; i < (int)(blockDim.x >> 6); ++i) tot += red_s[i];
-    const float scale = (kind == 0 ? A.q_scale : A.k_scale) * rsqrtf(tot / (float)A.Dk + A.eps);
+    const int nw = (int)(blockDim.x >> 6);
+    float tot;
+    if (nw == 4) tot = __fadd_rn(__fadd_rn(red_s[0], red_s[1]), __fadd_rn(red_s[2], red_s[3]));
+    else {
+        tot = red_s[0];
+        for (int i = 1; i < nw; ++i) tot = __fadd_rn(tot, red_s[i]);
+    }
+    const float scale = gdn_norm_scale(tot, A.Dk, A.eps, kind == 0 ? A.q_scale : A.k_scale);
     if (on) {
         Elem* dst = reinterpret_cast<Elem*>(kind == 0 ? A.q : A.k);
         dst[(((size_t)b * A.T + t) * A.Hk + head) * A.Dk + tid] = from_float<Elem>(y * scale);
@@ -187,9 +190,10 @@ extern "C" int dflash_gdn_finish(void* stream, const void* y, const void* gate, 
     A.rows = (int)rows; A.Dv = Dv; A.silu_gate = gate_kind;
     dim3 grid((unsigned)((rows + 3) / 4));
     hipStream_t st = (hipStream_t)stream;
-    if (in_dtype == DFLASH_F32) hipLaunchKernelGGL(gdn_finish_kernel<float>, grid, dim3(256), 0, st, A);
-    else if (in_dtype == DFLASH_BF16) hipLaunchKernelGGL(gdn_finish_kernel<bf16_t>, grid, dim3(256), 0, st, A);
-    else hipLaunchKernelGGL(gdn_finish_kernel<f16_t>, grid, dim3(256), 0, st, A);
+    LaunchBracket br(DFLASH_KERNEL_GDN_FINISH, st);
+    if (in_dtype == DFLASH_F32) br.launch(gdn_finish_kernel<float>, grid, dim3(256), 0, A);
+    else if (in_dtype == DFLASH_BF16) br.launch(gdn_finish_kernel<bf16_t>, grid, dim3(256), 0, A);
+    else br.launch(gdn_finish_kernel<f16_t>, grid, dim3(256), 0, A);
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
 }

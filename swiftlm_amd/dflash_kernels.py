@@ -189,6 +189,63 @@ class DFlashKernels:
         return out
 
     @staticmethod
+    def gdn_layer(mixed_qkv: torch.Tensor, conv_state: Optional[torch.Tensor], conv_weight: torch.Tensor,
+                  a_logits: torch.Tensor, b_logits: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
+                  state: torch.Tensor, Hk: int, Hv: int, Dk: int, Dv: int, q_scale: float, k_scale: float,
+                  eps: float = 1e-6, gate: Optional[torch.Tensor] = None, norm_weight: Optional[torch.Tensor] = None,
+                  norm_eps: float = 1e-6, gate_kind: str = "sigmoid", want_intermediates: bool = False):
+        """The body of a GatedDelta layer between its projections (KimiLinearDFlash.swift:351-378) in one
+        call: ``gdn_prepare`` -> ``gated_delta_kernel_with_tape`` -> ``gdn_finish`` with the pre-ops done
+        inside the forward kernel.  Returns a dict: ``out`` (None without ``gate``), ``y``, ``state``,
+        ``tape``, ``k``, ``g`` (what ``record_tape`` keeps), ``conv_state``, and with
+        ``want_intermediates`` also ``q``, ``v``, ``beta``.  Raises DFlashUnsupported outside the verify
+        block's case (float32 state, scalar gate, K == 4, T <= 16), where the three calls apply."""
+        _dev(mixed_qkv, conv_state, conv_weight, a_logits, b_logits, a_log, dt_bias, state, gate, norm_weight)
+        B, T, C = mixed_qkv.shape
+        if C != 2 * Hk * Dk + Hv * Dv:
+            raise DFlashError(f"gdn_layer: {C} channels, expected 2*{Hk}*{Dk} + {Hv}*{Dv}")
+        if a_logits.dim() != 3:
+            raise DFlashUnsupported("gdn_layer: one decay per head and step only (a_logits [B,T,Hv])")
+        if state.dtype != torch.float32:
+            raise DFlashUnsupported("gdn_layer: float32 state only")
+        K = int(conv_weight.shape[1])
+        dt = mixed_qkv.dtype
+        dv = mixed_qkv.device
+        x = mixed_qkv.contiguous()
+        w = conv_weight.to(dt).contiguous()
+        st = None if conv_state is None else conv_state.to(dt).contiguous()
+        a = a_logits.to(dt).contiguous()
+        bl = b_logits.to(dt).contiguous()
+        al = a_log.float().contiguous()
+        db = dt_bias.float().contiguous().reshape(-1)
+        state = state.contiguous()
+        k = torch.empty(B, T, Hk, Dk, dtype=dt, device=dv)
+        g = torch.empty(B, T, Hv, dtype=dt, device=dv)
+        y = torch.empty(B, T, Hv, Dv, dtype=dt, device=dv)
+        tape = torch.empty(B, T, Hv, Dv, dtype=torch.float32, device=dv)
+        new_state = torch.empty_like(state)
+        new_conv = torch.empty(B, K - 1, C, dtype=dt, device=dv)
+        q = torch.empty_like(k) if want_intermediates else None
+        v = torch.empty_like(y) if want_intermediates else None
+        beta = torch.empty_like(g) if want_intermediates else None
+        out = zg = nw = None
+        if gate is not None:
+            if norm_weight is None or gate.shape != y.shape or norm_weight.shape != (Dv,):
+                raise DFlashError("gdn_layer: gate must be [B,T,Hv,Dv] and come with norm_weight [Dv]")
+            zg, nw = gate.to(dt).contiguous(), norm_weight.to(dt).contiguous()
+            out = torch.empty_like(y)
+        rc = _lib.load().dflash_gdn_layer(
+            _stream(), _ptr(x), _ptr(st), _ptr(w), _ptr(a), _ptr(bl), _ptr(al), _ptr(db), _code(x),
+            float(q_scale), float(k_scale), float(eps), _ptr(state), _ptr(new_state), _ptr(k), _ptr(g), _ptr(tape),
+            _ptr(new_conv), _ptr(y), _ptr(zg), _ptr(nw), float(norm_eps), {"sigmoid": 0, "silu": 1}[gate_kind],
+            _ptr(out), _ptr(q), _ptr(v), _ptr(beta), B, T, Hk, Hv, Dk, Dv, K)
+        _lib.check(rc, "gdn_layer")
+        res = dict(out=out, y=y, state=new_state, tape=tape, k=k, g=g, conv_state=new_conv)
+        if want_intermediates:
+            res.update(q=q, v=v, beta=beta)
+        return res
+
+    @staticmethod
     def batched_sdpa_2pass(queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, scale: float,
                            mask: Optional[torch.Tensor] = None, *, return_lse: bool = False,
                            kv_len: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None):

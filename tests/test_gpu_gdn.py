@@ -330,3 +330,68 @@ def test_gdn_finish_matches_oracle(gpu_lib, shape, in_dt, kind):
     torch.cuda.synchronize()
     tol = dict(rtol=2e-5, atol=2e-6) if in_dt == "f32" else LOWP_TOL
     np.testing.assert_allclose(host(got), O.gdn_finish(y, z, w, 1e-6, kind), **tol)
+
+
+# ---- one-launch layer: pre-ops inside the forward kernel (KimiLinearDFlash.swift:351-378) ----
+
+@pytest.mark.parametrize("cfg", [(1, 16, 16, 32, 128, 128), (2, 5, 2, 4, 64, 48), (1, 2, 1, 2, 256, 32),
+                                 (1, 1, 2, 2, 128, 16), (1, 16, 4, 8, 64, 64)],
+                         ids=["qwen3next_block", "short_block_b2", "T_shorter_than_window_dk256", "single_step", "dk64"])
+@pytest.mark.parametrize("in_dt", ["bf16", "f32", "f16"])
+@pytest.mark.parametrize("carry", [True, False], ids=["conv_state", "no_conv_state"])
+def test_gdn_layer_equals_prepare_forward_finish_bitwise(gpu_lib, cfg, in_dt, carry):
+    """dflash_gdn_layer against the three calls it replaces: every output bit for bit, and the three-call
+    result against the oracle (so the equality is not two wrong answers agreeing)."""
+    from swiftlm_amd import DFlashKernels as K
+
+    B, T, Hk, Hv, Dk, Dv = cfg
+    Kc = 4
+    d = _prep_inputs(B * 1000 + T * 10 + Dk, B, T, Hk, Hv, Dk, Dv, Kc, False)
+    rd = {"f32": lambda a: a, "bf16": O.round_to_bf16, "f16": lambda a: a.astype(np.float16).astype(np.float32)}[in_dt]
+    x, st, w, a, bl = (dev(rd(d[n]), in_dt) for n in ("x", "state", "w", "a", "b"))
+    if not carry:
+        st = None
+    rng = np.random.default_rng(5)
+    s0 = dev(0.1 * rng.standard_normal((B, Hv, Dv, Dk)).astype(np.float32))
+    z = dev(rd((rng.standard_normal((B, T, Hv, Dv)) * 2).astype(np.float32)), in_dt)
+    nw = dev(rd((1 + 0.1 * rng.standard_normal(Dv)).astype(np.float32)), in_dt)
+    sc = dict(q_scale=1.0 / Dk, k_scale=Dk ** -0.5)
+
+    q, k, v, g, beta, conv1 = K.gdn_prepare(x, st, w, a, bl, dev(d["a_log"]), dev(d["dt_bias"]), Hk, Hv, Dk, Dv, **sc)
+    y, s1, tape = K.gated_delta_kernel_with_tape(q, k, v, g, beta, s0)
+    out = K.gdn_finish(y, z, nw, 1e-6, "silu")
+    r = K.gdn_layer(x, st, w, a, bl, dev(d["a_log"]), dev(d["dt_bias"]), s0, Hk, Hv, Dk, Dv, **sc, gate=z, norm_weight=nw,
+                    norm_eps=1e-6, gate_kind="silu", want_intermediates=True)
+    torch.cuda.synchronize()
+    for name, want in (("q", q), ("k", k), ("v", v), ("g", g), ("beta", beta), ("conv_state", conv1), ("y", y),
+                       ("state", s1), ("tape", tape), ("out", out)):
+        assert torch.equal(r[name], want), name
+    # without the optional outputs and without a gate: same recurrence results
+    r2 = K.gdn_layer(x, st, w, a, bl, dev(d["a_log"]), dev(d["dt_bias"]), s0, Hk, Hv, Dk, Dv, **sc)
+    torch.cuda.synchronize()
+    assert r2["out"] is None
+    for name in ("y", "state", "tape", "k", "g", "conv_state"):
+        assert torch.equal(r2[name], r[name]), name
+    # and the three calls against the oracle
+    want = O.gdn_prepare(host(x), None if st is None else host(st), host(w), host(a), host(bl), d["a_log"], d["dt_bias"],
+                         Hk, Hv, Dk, Dv, **sc)
+    tol = dict(rtol=2e-5, atol=2e-6) if in_dt == "f32" else LOWP_TOL
+    for name in ("q", "k", "v", "g", "beta"):
+        np.testing.assert_allclose(host(r[name]), want[name], err_msg=name, **tol)
+    yw, sw, tw = O.gated_delta_ops_with_tape(host(q), host(k), host(v), host(g), host(beta), host(s0), dtype=np.float64)
+    np.testing.assert_allclose(host(r["state"]), sw, **STATE_TOL)
+    np.testing.assert_allclose(host(r["tape"]), tw, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(host(r["y"]), yw, **(dict(rtol=1e-4, atol=1e-5) if in_dt == "f32" else LOWP_TOL))
+    np.testing.assert_allclose(host(r["out"]), O.gdn_finish(host(y), host(z), host(nw), 1e-6, "silu"), **tol)
+
+
+def test_gdn_layer_reports_unsupported_outside_the_verify_block(gpu_lib):
+    from swiftlm_amd import DFlashKernels as K
+    from swiftlm_amd.dflash_kernels import DFlashUnsupported
+
+    B, Hk, Hv, Dk, Dv = 1, 2, 2, 128, 32
+    for T, Kc in ((17, 4), (8, 3)):
+        d = _prep_inputs(3, B, T, Hk, Hv, Dk, Dv, Kc, False)
+        args = [dev(d[n], "bf16") for n in ("x", "state", "w", "a", "b")] + [dev(d["a_log"]), dev(d["dt_bias"])]
+        with pytest.raises(DFlashUnsupported):
+            K.gdn_layer(*args, torch.zeros(B, Hv, Dv, Dk, device="cuda"), Hk, Hv, Dk, Dv, q_scale=1.0, k_scale=1.0)
