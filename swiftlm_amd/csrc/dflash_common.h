@@ -209,4 +209,21 @@ template <int LANES> __device__ __forceinline__ float butterfly_sum(float x) {
     return x;
 }
 
+// The same butterfly for the maximum (order does not matter for a maximum; this is only the fast path: DPP and
+// lane swaps instead of six LDS permutes).
+template <int CTRL> __device__ __forceinline__ float dpp_max(float x) {
+    int y = __builtin_amdgcn_update_dpp(__float_as_int(x), __float_as_int(x), CTRL, 0xf, 0xf, false);
+    return fmaxf(x, __int_as_float(y));
+}
+__device__ __forceinline__ float wave_max(float x) {
+    x = dpp_max<0xB1>(x);
+    x = dpp_max<0x4E>(x);
+    x = dpp_max<0x141>(x);
+    x = dpp_max<0x140>(x);
+    auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    auto r2 = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r2[0]), __uint_as_float(r2[1]));
+}
+
 }  // namespace dflash

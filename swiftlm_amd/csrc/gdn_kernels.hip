@@ -85,6 +85,10 @@ __global__ __launch_bounds__(kThreads) void tape_replay_kernel(ReplayBatch P, Re
     __shared__ float d_s[TC][ROWS];
     __shared__ int on_s[TC];
 
+    // the scalar arguments in one burst of loads (the per-layer pointer tables are indexed by the layer and stay lazy)
+    asm volatile("" ::"s"(A.mask), "s"(A.steps_dev), "s"(A.verify_ids), "s"(A.posterior), "s"(A.start_inout), "s"(A.out4),
+                 "s"(A.V), "s"(A.mask_dtype), "s"(A.tape_dtype), "s"(A.in_dtype), "s"(A.steps), "s"(A.skip_if_full),
+                 "s"(A.T_tape), "s"(A.Hk), "s"(A.Hv), "s"(A.Dv));
     const int layer = blockIdx.z;
     const int bh = blockIdx.y;
     const int b = bh / A.Hv, hv = bh % A.Hv;

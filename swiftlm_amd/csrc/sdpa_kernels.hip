@@ -208,6 +208,13 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t smem_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
+    // All kernel arguments in one burst of scalar loads: fetched where they are first used they arrive in three
+    // dependent rounds (with the device-side length in the middle), each a trip to memory ahead of the first tile.
+    asm volatile("" ::"s"(A.q), "s"(A.k), "s"(A.v), "s"(A.k_new), "s"(A.v_new), "s"(A.k_cache), "s"(A.v_cache), "s"(A.part_o),
+                 "s"(A.part_m), "s"(A.part_l), "s"(A.kv_len_dev), "s"(A.mask), "s"(A.kv_batch_stride), "s"(A.kv_head_stride));
+    asm volatile("" ::"s"(A.scale_log2), "s"(A.Hq), "s"(A.Hk), "s"(A.G), "s"(A.N), "s"(A.S), "s"(A.groups_per_kv),
+                 "s"(A.rows_total), "s"(A.len_bias), "s"(A.page_table), "s"(A.page_shift), "s"(A.table_stride), "s"(A.num_pages));
+
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -743,6 +750,7 @@ __global__ __launch_bounds__(kCombineThreads) void sdpa_combine_kernel(CombineAr
     __shared__ float red_s[kCombineThreads / 64];
     __shared__ float acc_s[NG][D];
 
+    asm volatile("" ::"s"(A.part_o), "s"(A.part_m), "s"(A.part_l), "s"(A.out), "s"(A.lse), "s"(A.S));   // one burst of argument loads
     const size_t row = blockIdx.x;
     const int tid = threadIdx.x;
     const float* pm = A.part_m + row * A.S;
@@ -751,7 +759,7 @@ __global__ __launch_bounds__(kCombineThreads) void sdpa_combine_kernel(CombineAr
     // global max
     float mx = -INFINITY;
     for (int s = tid; s < A.S; s += kCombineThreads) mx = fmaxf(mx, pm[s]);
-    for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    mx = wave_max(mx);
     if ((tid & 63) == 0) red_s[tid >> 6] = mx;
     __syncthreads();
     mx = fmaxf(fmaxf(red_s[0], red_s[1]), fmaxf(red_s[2], red_s[3]));
@@ -764,7 +772,7 @@ __global__ __launch_bounds__(kCombineThreads) void sdpa_combine_kernel(CombineAr
         w_s[s] = w;
         lsum += w;
     }
-    for (int o = 32; o >= 1; o >>= 1) lsum += __shfl_xor(lsum, o);
+    lsum = butterfly_sum<64>(lsum);
     if ((tid & 63) == 0) red_s[tid >> 6] = lsum;
     __syncthreads();
     lsum = red_s[0] + red_s[1] + red_s[2] + red_s[3];
