@@ -120,6 +120,14 @@ __device__ __forceinline__ void async_load_16B(const unsigned char* gbase, uint3
                  : "memory", "m0");
 }
 
+// The same without the non-temporal hint (Q, which every workgroup of the head re-reads).
+__device__ __forceinline__ void async_load_16B_plain(const unsigned char* gbase, uint32_t goff, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(goff), "s"(gbase), "s"(__builtin_amdgcn_readfirstlane(lds_base))
+                 : "memory", "m0");
+}
+
 // Tells the compiler a wave-uniform pointer is uniform (inline-assembly "s" operands need SGPRs).
 __device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char* p) {
     const uint64_t u = (uint64_t)p;
@@ -190,12 +198,14 @@ template <int D> struct SdpaLds {
     static constexpr int K_RING = Q_BYTES;
     static constexpr int V_RING = Q_BYTES + kRingSlots * KT;
     static constexpr int LPP = (kBN / RPI) / 2;              // load instructions per producer wave per K (or V) tile
-    static constexpr int QPP = (128 / RPI) / 2;              // ... for Q
     static constexpr int EROW = D * 2 + 16;                  // epilogue O row pitch, bytes
     static constexpr int EPI = 4 * 32 * EROW;
     static constexpr int RING_END = Q_BYTES + 2 * kRingSlots * KT;
     static constexpr int BYTES = RING_END > EPI ? RING_END : EPI;
 };
+
+// The t-th tile of a split: tiles are dealt in rows of S neighbouring tiles, one per split.
+__device__ __forceinline__ int tile_index(int split, int t, int S) { return t * S + split; }
 
 template <typename Tag, int D, bool MASKED, bool PAGED>
 __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaArgs A) {
@@ -235,7 +245,7 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
     auto load_entries = [&](int base) -> int {
         // no branch and no arithmetic on the value here: the wait for it then sits at its first use, not at the load
         const int nt_max = (A.N + kBN - 1) / kBN;
-        int tile = split + (base + lane) * A.S;
+        int tile = tile_index(split, base + lane, A.S);
         tile = tile < nt_max ? tile : nt_max - 1;
         return A.page_table[(size_t)b * A.table_stride + ((tile * kBN) >> A.page_shift)];
     };
@@ -246,7 +256,42 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
         }
     }
 
-    int Nb = A.kv_len_dev ? A.kv_len_dev[b] + A.len_bias : A.N;
+    // The device-side key count is requested here, through the scalar cache, and awaited below the Q requests: a
+    // scalar read counts on its own counter, so waiting for it does not wait for Q.  (Written as assembly because
+    // the compiler would wait where the read is issued; the register is not touched between the two statements.
+    // Without a device-side count a word of Q is read and dropped, which keeps the sequence free of branches.)
+    int len_raw;
+    {
+        const int32_t* lp = A.kv_len_dev ? A.kv_len_dev + b : reinterpret_cast<const int32_t*>(A.q);
+        asm volatile("s_load_dword %0, %1, 0x0" : "=s"(len_raw) : "s"(lp));
+    }
+    // Q does not depend on the key count, and the compute waves have nothing to do until the first tile lands: each
+    // asks for its own 32 rows (heads 2w, 2w+1 of the group; an absent head re-reads the group's first head, its rows
+    // are never stored) while the device-side count is still on its way and the producers get ready for K(t_begin).
+    // Swizzled like a K tile, at w * 32 rows of the Q area.
+    if (!producer) {
+        const int ld_rsub = lane / L::CPR, ld_pos = lane % L::CPR;
+        const unsigned char* qb = reinterpret_cast<const unsigned char*>(A.q) + ((size_t)b * A.Hq + hk * A.G + hg0) * kM * L::ROWB;
+        if (2 * wave + 1 < hcount) {                 // uniform: both heads present, the 32 rows are contiguous
+            const unsigned char* qw = uniform_ptr(qb + (size_t)wave * 32 * L::ROWB);
+#pragma unroll
+            for (int j = 0; j < 32 / L::RPI; ++j) {
+                const int row = j * L::RPI + ld_rsub;
+                async_load_16B_plain(qw, (uint32_t)(row * L::ROWB + ((ld_pos ^ (row & 15)) * 16)),
+                                     smem_lds + (wave * 32 + j * L::RPI) * L::ROWB);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 32 / L::RPI; ++j) {
+                const int row = wave * 32 + j * L::RPI + ld_rsub;
+                const int head = (row >> 4) < hcount ? (row >> 4) : 0;
+                async_load_16B_addr<false>(qb + (size_t)(head * kM + (row & 15)) * L::ROWB + ((ld_pos ^ (row & 15)) * 16),
+                                    smem_lds + (wave * 32 + j * L::RPI) * L::ROWB);
+            }
+        }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(len_raw));
+    int Nb = A.kv_len_dev ? len_raw + A.len_bias : A.N;
     Nb = Nb < kM ? kM : (Nb > A.N ? A.N : Nb);
     const int nt = (Nb + kBN - 1) / kBN;
     // Tiles are dealt round-robin: split s takes tiles s, s + S, s + 2S, ...  At any moment the workgroups of a KV
@@ -254,9 +299,10 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
     // apart, which the memory system serves faster.  Below, t counts this split's own tiles (0 .. t_end-1) and
     // key_of(t) is the first key of its t-th tile.
     const int t_begin = 0;
-    const int t_end = split < nt ? (nt - split + A.S - 1) / A.S : 0;
+    const int t_full = nt / A.S;                                   // rows of S tiles that every split takes part in
+    const int t_end = t_full + (tile_index(split, t_full, A.S) < nt ? 1 : 0);
     const int t_last = t_end - 1;
-    auto key_of = [&](int t) { return (split + t * A.S) * kBN; };
+    auto key_of = [&](int t) { return tile_index(split, t, A.S) * kBN; };
 
     const int cw = producer ? 0 : wave;                      // compute wave index (producers: unused)
     const int head_in_group = 2 * cw + (c >> 4);
@@ -284,25 +330,34 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
             return (size_t)key * L::ROWB;
         }
     };
-    // Fused append: keys Nb-16 .. Nb-1 are read from k_new / v_new, and one workgroup per KV head stores them
+    // Fused append: keys Nb-16 .. Nb-1 are read from k_new / v_new, and the workgroups of the KV head store them
     // into the cache rows they stand for (paged: the 16 rows may straddle a page, so every row looks its page up).
-    // The copy is done by the compute waves, which have nothing to do until the first tile lands, of the LAST split,
-    // which never holds more tiles than the others: it stays off the launch's critical path.
+    // The copy is spread over all splits of the KV head (done whole by one workgroup it was four dependent round trips
+    // in that workgroup, which then finished last of the launch).
     const bool fused = A.k_new != nullptr;
     const int cache_rows = fused ? Nb - kM : Nb;       // keys below this index are read from the cache
     const unsigned char* knew = reinterpret_cast<const unsigned char*>(A.k_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
     const unsigned char* vnew = reinterpret_cast<const unsigned char*>(A.v_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
-    if (fused && A.k_cache && split == A.S - 1 && hg0 == 0 && !producer) {
+    if (fused && A.k_cache && hg0 == 0 && wave == 0) {
+        // 16-byte pieces of the block's rows, dealt evenly over the splits of the KV head: a handful per workgroup,
+        // read and written by the first compute wave in one round trip.
+        const int pieces = kM * L::CPR;
+        const int per = (pieces + A.S - 1) / A.S;
         const u32x4_t* ksrc = reinterpret_cast<const u32x4_t*>(knew);
         const u32x4_t* vsrc = reinterpret_cast<const u32x4_t*>(vnew);
-        for (int i = tid; i < kM * L::CPR; i += 4 * 64) {
-            const size_t off = head_off + row_off(cache_rows + i / L::CPR) + (size_t)(i % L::CPR) * 16;
-            *reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.k_cache) + off) = ksrc[i];
-            *reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.v_cache) + off) = vsrc[i];
+        for (int i0 = 0; i0 < per; i0 += 64) {
+            const int i = split * per + i0 + lane;
+            if (i0 + lane < per && i < pieces) {
+                const u32x4_t kx = ksrc[i], vx = vsrc[i];
+                const size_t off = head_off + row_off(cache_rows + i / L::CPR) + (size_t)(i % L::CPR) * 16;
+                *reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.k_cache) + off) = kx;
+                *reinterpret_cast<u32x4_t*>(reinterpret_cast<unsigned char*>(A.v_cache) + off) = vx;
+            }
         }
     }
 
     if (t_begin >= t_end) {   // empty split: tell the combine kernel to ignore it
+        wait_vmcnt<0>();                             // the Q requests must have landed before the wave ends
         if (row_valid && h == 0) {
             A.part_m[row_id * A.S + split] = -INFINITY;
             A.part_l[row_id * A.S + split] = 0.f;
@@ -374,38 +429,18 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
         auto group_loads = [&](int t) { return (t < t_end ? L::LPP : 0) + (t + 1 < t_end ? L::LPP : 0); };
 
         if constexpr (PAGED) asm volatile("" : "+v"(ent_cur), "+v"(ent_nxt));   // both gathers have landed from here on
-        {
-            const size_t o0 = tile_off(t_begin), o1 = tile_off(t_begin + 1);
-            issue_k(t_begin, o0);
-            // Q: 32 rows per compute wave (heads 2w, 2w+1 of the group), swizzled like a K tile, at w * 32 rows of the
-            // Q area; an absent head re-reads the group's first head (its rows are never stored).  Requested right
-            // behind the first K tile: the first scores need both, and nothing else should queue ahead of them.
-            // (Requested by the compute waves instead, Q lands behind the producers' whole opening burst.)
-            {
-                const unsigned char* qb = reinterpret_cast<const unsigned char*>(A.q) + ((size_t)b * A.Hq + hk * A.G + hg0) * kM * L::ROWB;
-#pragma unroll
-                for (int j = 0; j < L::QPP; ++j) {
-                    const int row = (2 * j + pw) * L::RPI + ld_rsub;           // 0..127 over the four compute waves
-                    const int head = (row >> 4) < hcount ? (row >> 4) : 0;
-                    async_load_16B_addr<false>(qb + (size_t)(head * kM + (row & 15)) * L::ROWB + ((ld_pos ^ (row & 15)) * 16),
-                                        smem_lds + (2 * j + pw) * L::RPI * L::ROWB);
-                }
-            }
-            issue_v(t_begin, o0); issue_k(t_begin + 1, o1);     // group t_begin
-            issue_v(t_begin + 1, o1);                           // group t_begin + 1 ...
-        }
+        // Opening: only K(t_begin) (Q is already on its way) stands between the compute waves and their first
+        // scores, so the first barrier waits for just these; the next two groups are requested behind it, while the
+        // compute waves already work on tile t_begin.
+        const size_t o0 = tile_off(t_begin), o1 = tile_off(t_begin + 1);
+        issue_k(t_begin, o0);
+        wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();                       // Q and K(t_begin) are in LDS
+        issue_v(t_begin, o0); issue_k(t_begin + 1, o1);     // group t_begin
+        issue_v(t_begin + 1, o1);                           // group t_begin + 1 ...
         size_t off_v = tile_off(t_begin + 2);                   // tile whose V the next iteration requests
         issue_k(t_begin + 2, off_v);                            // ... and its K
         size_t off_k = tile_off(t_begin + 3);                   // tile whose K the next iteration requests
-        {
-            const int later = group_loads(t_begin) + group_loads(t_begin + 1);     // 0 .. 4 * LPP
-            if (later >= 4 * L::LPP) wait_vmcnt<4 * L::LPP>();
-            else if (later >= 3 * L::LPP) wait_vmcnt<3 * L::LPP>();
-            else if (later >= 2 * L::LPP) wait_vmcnt<2 * L::LPP>();
-            else if (later >= L::LPP) wait_vmcnt<L::LPP>();
-            else wait_vmcnt<0>();
-        }
-        __builtin_amdgcn_s_barrier();                       // Q and K(t_begin) are in LDS
         for (int t = t_begin; t <= t_last; ++t) {
             const int later = group_loads(t + 1);
             if (later >= 2 * L::LPP) wait_vmcnt<2 * L::LPP>();
@@ -642,6 +677,7 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
         }
     };
 
+    wait_vmcnt<0>();                                // this wave's Q rows have landed
     __builtin_amdgcn_s_barrier();                   // Q and K(t_begin) are in LDS
     if (wave_active) {
         qk_tile(t_begin);
