@@ -592,16 +592,18 @@ template <int QUAD_LANE> __device__ __forceinline__ float quad_broadcast(float x
 }
 
 // Steps S..15 of the unit-triangular solve for one state row held by a quad (lane q owns steps 4q..4q+3).
+// Every lane of the quad sees every delta; lane q keeps those of its own four steps in `mine` (a select per step,
+// no branch) for the store that follows.
 template <int S> struct SolveStep {
     static __device__ __forceinline__ void run(float (&acc)[4], const float4 (&arow)[16], const float (&bet)[16],
-                                               float (&dv)[16]) {
+                                               float (&mine)[4], const int q) {
         const float d = quad_broadcast<S / 4>(bet[S] * acc[S % 4]);
-        dv[S] = d;
+        mine[S % 4] = q == S / 4 ? d : mine[S % 4];
         acc[0] = fmaf(-arow[S].x, d, acc[0]);
         acc[1] = fmaf(-arow[S].y, d, acc[1]);
         acc[2] = fmaf(-arow[S].z, d, acc[2]);
         acc[3] = fmaf(-arow[S].w, d, acc[3]);
-        if constexpr (S + 1 < 16) SolveStep<S + 1>::run(acc, arow, bet, dv);
+        if constexpr (S + 1 < 16) SolveStep<S + 1>::run(acc, arow, bet, mine, q);
     }
 };
 
@@ -869,6 +871,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         // ---- [S_0 ; k] x [k | q]^T, wave w contracting channels w*DK/4 .. +DK/4-1 ----
         // A 32x32x2 fp32 MFMA takes lane l's a as row l%32, contraction index l/32 (b alike), so a float4
         // per lane feeds four MFMAs whose index pairs are {e, 4+e} of an 8-channel group.
+        float G = 1.f;                      // decay product of the pair (s, t) = (ts, tt)
         {
             f32x16v acc;
 #pragma unroll
@@ -883,13 +886,24 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
                 acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.z, b4.z, acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.w, b4.w, acc, 0, 0, 0);
             }
+            // The decay products run in the shadow of the MFMAs (the matrix pipe is busy for a thousand cycles after
+            // the last one is issued): all 16 decays are read unconditionally, four at a time, and selected in
+            // registers -- a conditional read per step costs an exec-mask round trip each.
+            __builtin_amdgcn_sched_barrier(0);
+            {
+                float gj[kChunkSteps];
+#pragma unroll
+                for (int j4 = 0; j4 < kChunkSteps; j4 += 4) {
+                    const float4 g4 = *reinterpret_cast<const float4*>(&L.g[j4]);
+                    gj[j4] = g4.x; gj[j4 + 1] = g4.y; gj[j4 + 2] = g4.z; gj[j4 + 3] = g4.w;
+                }
+#pragma unroll
+                for (int j = 1; j < kChunkSteps; ++j) G *= (j > ts && j <= tt) ? gj[j] : 1.f;
+            }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int v = 0; v < 16; ++v) L.red[w][8 * (v / 4) + 4 * (lane / 32) + (v % 4)][lane % 32] = acc[v];
         }
-        // decay products for the pair (s, t) = (ts, tt)
-        float G = 1.f;
-#pragma unroll
-        for (int j = 1; j < kChunkSteps; ++j) G *= (j > ts && j <= tt) ? L.g[j] : 1.f;
         __syncthreads();
         // sum the four partial products: the S_0 half (16 x 32) as two entries per thread, the k half
         // straight into the coefficient tables of the pair (ts, tt)
@@ -909,7 +923,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         // betas, the LDS stores of delta) is kept off it.
         if (w == 0) {
             const int r = lane / 4, q = lane % 4;
-            float acc[4], bet[16], dv[16];
+            float acc[4], bet[16], mine[4] = {0.f, 0.f, 0.f, 0.f};
             float4 arow[16];
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[e] = fmaf(-L.gam[4 * q + e], L.p[r][4 * q + e], L.v[4 * q + e][r]);
@@ -918,12 +932,9 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
                 arow[s] = *reinterpret_cast<const float4*>(&L.a[s][4 * q]);
                 bet[s] = L.beta[s];
             }
-            SolveStep<0>::run(acc, arow, bet, dv);
+            SolveStep<0>::run(acc, arow, bet, mine, q);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float d = q == 0 ? dv[e] : q == 1 ? dv[4 + e] : q == 2 ? dv[8 + e] : dv[12 + e];
-                L.dl[4 * q + e][r] = d;
-            }
+            for (int e = 0; e < 4; ++e) L.dl[4 * q + e][r] = mine[e];
         }
         __syncthreads();
 
