@@ -783,52 +783,61 @@ __global__ __launch_bounds__(kCombineThreads) void sdpa_combine_kernel(CombineAr
     constexpr int NG = kCombineThreads / TPG;         // split groups walking the partials in parallel
     constexpr int UNROLL = 16;                     // row loads in flight per thread: one round trip for S <= 16 * NG
     __shared__ float w_s[kMaxSplits];
-    __shared__ float red_s[kCombineThreads / 64];
+    __shared__ float redm_s[kCombineThreads / 64], reds_s[kCombineThreads / 64];
     __shared__ float acc_s[NG][D];
+    static_assert(kMaxSplits <= 2 * kCombineThreads, "a thread holds the statistics of at most two splits");
 
     asm volatile("" ::"s"(A.part_o), "s"(A.part_m), "s"(A.part_l), "s"(A.out), "s"(A.lse), "s"(A.S));   // one burst of argument loads
     const size_t row = blockIdx.x;
     const int tid = threadIdx.x;
     const float* pm = A.part_m + row * A.S;
     const float* pl = A.part_l + row * A.S;
+    const int grp = tid / TPG, d8 = (tid % TPG) * 8;
+    const uint16_t* po = A.part_o + row * D + d8;
+
+    // Everything the row needs is requested in one go: the statistics of this thread's splits (tid and, beyond 256
+    // splits, tid + 256; addresses clamped, values dropped) and the first UNROLL partial rows of its group.  Asked
+    // for one after the other -- maxima, then sums, then rows -- they are three dependent trips to memory.
+    const int sa = tid < A.S ? tid : A.S - 1, sb = tid + kCombineThreads < A.S ? tid + kCombineThreads : A.S - 1;
+    float m0 = pm[sa], m1 = pm[sb];
+    const float l0 = pl[sa], l1 = pl[sb];
+    u32x4_t raw[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const int sp = grp + u * NG;
+        // Loaded without looking at the weight (a branch per load makes the loads wait for one another); the rows of
+        // empty splits hold no data, whatever was read from them is dropped below.
+        raw[u] = *reinterpret_cast<const u32x4_t*>(po + (size_t)(sp < A.S ? sp : 0) * gridDim.x * D);
+    }
+    if (tid >= A.S) m0 = -INFINITY;
+    if (tid + kCombineThreads >= A.S) m1 = -INFINITY;
 
     // global max
-    float mx = -INFINITY;
-    for (int s = tid; s < A.S; s += kCombineThreads) mx = fmaxf(mx, pm[s]);
-    mx = wave_max(mx);
-    if ((tid & 63) == 0) red_s[tid >> 6] = mx;
+    float mx = wave_max(fmaxf(m0, m1));
+    if ((tid & 63) == 0) redm_s[tid >> 6] = mx;
     __syncthreads();
-    mx = fmaxf(fmaxf(red_s[0], red_s[1]), fmaxf(red_s[2], red_s[3]));
+    mx = fmaxf(fmaxf(redm_s[0], redm_s[1]), fmaxf(redm_s[2], redm_s[3]));
+    // weights and denominator (the partial rows are O / l: weight by l)
+    const float w0 = m0 == -INFINITY ? 0.f : fast_exp2(m0 - mx) * l0;
+    const float w1 = m1 == -INFINITY ? 0.f : fast_exp2(m1 - mx) * l1;
+    if (tid < A.S) w_s[tid] = w0;
+    if (tid + kCombineThreads < A.S) w_s[tid + kCombineThreads] = w1;
+    float lsum = butterfly_sum<64>(w0 + w1);
+    if ((tid & 63) == 0) reds_s[tid >> 6] = lsum;
     __syncthreads();
-    // weights and denominator
-    float lsum = 0.f;
-    for (int s = tid; s < A.S; s += kCombineThreads) {
-        const float m = pm[s];
-        const float w = m == -INFINITY ? 0.f : fast_exp2(m - mx) * pl[s];   // the partial rows are O / l: weight by l
-        w_s[s] = w;
-        lsum += w;
-    }
-    lsum = butterfly_sum<64>(lsum);
-    if ((tid & 63) == 0) red_s[tid >> 6] = lsum;
-    __syncthreads();
-    lsum = red_s[0] + red_s[1] + red_s[2] + red_s[3];
+    lsum = reds_s[0] + reds_s[1] + reds_s[2] + reds_s[3];
 
     // weighted sum of the partial rows: group grp takes splits grp, grp + NG, ...
-    const int grp = tid / TPG, d8 = (tid % TPG) * 8;
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-    const uint16_t* po = A.part_o + row * D + d8;
     for (int s0 = grp; s0 < A.S; s0 += NG * UNROLL) {
-        u32x4_t raw[UNROLL];
         float w[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            const int s = s0 + u * NG;
-            w[u] = s < A.S ? w_s[s] : 0.f;
-            // Loaded without looking at the weight (a branch per load makes the loads wait for one another); the rows of
-            // empty splits hold no data, whatever was read from them is dropped below.
-            raw[u] = *reinterpret_cast<const u32x4_t*>(po + (size_t)(s < A.S ? s : 0) * gridDim.x * D);
+            const int sp = s0 + u * NG;
+            w[u] = sp < A.S ? w_s[sp] : 0.f;
+            if (s0 != grp) raw[u] = *reinterpret_cast<const u32x4_t*>(po + (size_t)(sp < A.S ? sp : 0) * gridDim.x * D);
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
