@@ -396,6 +396,79 @@ def aux_gdn_layer(lib, cfg, n_layers=36, reps=30):
     return res
 
 
+def side_config(lib, name, reps=40):
+    """BASELINE configs 1-3 (parity-test cases, not the headline number), timed so that their kernels can be
+    profiled at their own shapes: every launch carries events on its dispatch; medians in microseconds.
+      config1  tape replay at the Qwen3-Next shape, 36 layers launched one by one, n ~ Geometric(0.25) in [1,16]
+      config2  block-causal attention, L=4096, Hq=16 Hkv=2 D=256 bf16
+      config3  the same at L=40960 and L=102400, and a ragged batch of 4 sequences with L ~ U[8K,64K]"""
+    import torch
+    from swiftlm_amd import DFlashKernels as K, _lib
+
+    dev, bf = "cuda", torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(21)
+    rn = lambda *shape: torch.randn(*shape, generator=g, device=dev)
+    out = {"metric": "dflash_side_config_us", "workload": name, "unit": "us", "data": "synthetic", "dtype": "bf16"}
+
+    def timed(kernel_id, calls):
+        for c in calls[:3]:
+            c()
+        ev = HipEvents()
+        for c in calls:
+            a, b = ev.pair()
+            _lib.check(lib.dflash_profile_next_launch(kernel_id, a, b), "profile_next_launch")
+            c()
+        torch.cuda.synchronize()
+        d = np.array(ev.durations_us())
+        ev.destroy()
+        return {"median_us": round(float(np.median(d)), 2), "min_us": round(float(d.min()), 2), "launches": len(d)}
+
+    if name == "config1":
+        B, T, Hk, Hv, Dk, Dv, n_layers = 1, 16, 16, 32, 128, 128, 36
+        rng = np.random.default_rng(3)
+        ns = [int(min(rng.geometric(0.25), T)) for _ in range(n_layers)]
+        layers = [dict(tape=rn(B, T, Hv, Dv), k=torch.nn.functional.normalize(rn(B, T, Hk, Dk), dim=-1).to(bf),
+                       g=torch.rand(B, T, Hv, generator=g, device=dev).to(bf), s=0.1 * rn(B, Hv, Dv, Dk)) for _ in range(n_layers)]
+        calls = [(lambda l=l, n=n: K.tape_replay_kernel(l["tape"][:, :n].contiguous(), l["k"][:, :n].contiguous(),
+                                                        l["g"][:, :n].contiguous(), l["s"])) for l, n in zip(layers, ns)]
+        r = timed(_lib.KERNEL_TAPE_REPLAY, calls * 2)
+        nbytes = [2 * Hv * Dv * Dk * 4 + n * (Hv * Dv * 4 + Hk * Dk * 2 + Hv * 2) for n in ns]
+        r["algorithmic_bytes_mean"] = int(np.mean(nbytes))
+        r["gbs"] = round(np.mean(nbytes) / r["median_us"] / 1e3, 1)
+        r["accepted_n"] = ns
+        out["tape_replay_single_layer"] = r
+        # the same 36 layers the way the verify step does them: one batched launch
+        st_in, st_out = [l["s"] for l in layers], [torch.empty_like(l["s"]) for l in layers]
+        n_dev = torch.tensor([4], dtype=torch.int32, device=dev)
+        calls = [lambda: K.tape_replay_batched([l["tape"] for l in layers], [l["k"] for l in layers], [l["g"] for l in layers],
+                                               st_in, st_out, 4, steps_dev=n_dev)] * 12
+        r = timed(_lib.KERNEL_TAPE_REPLAY, calls)
+        r["us_per_layer"] = round(r["median_us"] / n_layers, 3)
+        out["tape_replay_batched_36_layers_n4"] = r
+    else:
+        Hq, Hk, D = 16, 2, 256
+        cases = {"config2": [("L4096", [4096])],
+                 "config3": [("L40960", [40960]), ("L102400", [102400]),
+                             ("ragged_batch4", [int(x) for x in np.random.default_rng(4).integers(8192, 65537, 4)])]}[name]
+        for label, Ls in cases:
+            B, N = len(Ls), max(Ls) + 16
+            nset = max(2, min(8, int(600e6 // (B * Hk * N * D * 4))))          # rotate through ~600 MB so nothing stays cached
+            sets = [(rn(B, Hq, 16, D).to(bf), rn(B, Hk, N, D).to(bf), rn(B, Hk, N, D).to(bf)) for _ in range(nset)]
+            kv_len = torch.tensor([l + 16 for l in Ls], dtype=torch.int32, device=dev) if B > 1 else None
+            ws = torch.empty(K.sdpa_workspace_bytes(B, Hq, Hk, 16, N, D), dtype=torch.uint8, device=dev)
+            calls = [(lambda q=q, k=k, v=v: K.batched_sdpa_2pass(q, k, v, D ** -0.5, kv_len=kv_len, workspace=ws))
+                     for q, k, v in sets] * max(1, reps // nset)
+            nbytes = sum(2 * Hq * 16 * D * 2 + 2 * Hk * (l + 16) * D * 2 + Hq * 16 * 4 for l in Ls)
+            part = timed(_lib.KERNEL_SDPA_PARTIAL, calls)
+            comb = timed(_lib.KERNEL_SDPA_COMBINE, calls)
+            out[label] = {"context": Ls, "algorithmic_bytes": nbytes, "sdpa_partial": part, "sdpa_combine": comb,
+                          "partial_gbs": round(nbytes / part["median_us"] / 1e3, 1),
+                          "partial_frac_of_hbm_peak": round(nbytes / part["median_us"] / 1e3 / HBM_PEAK_GBS, 4),
+                          "both_gbs": round(nbytes / (part["median_us"] + comb["median_us"]) / 1e3, 1)}
+            del sets, ws
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -410,6 +483,9 @@ def main():
     ap.add_argument("--page-size", type=int, default=0,
                     help="keep the attention layers' K/V in paged pools with pages of this many keys (0: dense caches, "
                          "the configuration the headline number is quoted on)")
+    ap.add_argument("--workload", default="config4", choices=["config4", "config1", "config2", "config3"],
+                    help="config4 (default) is the benchmark; config1-3 time BASELINE's other configurations at their own "
+                         "shapes (parity-test cases; a separate JSON line, not the headline metric)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy, the known-size kernel the rocprof byte counters are scaled by")
     args = ap.parse_args()
@@ -426,6 +502,10 @@ def main():
     torch.cuda.set_device(0)
     lib = _lib.load()
     _lib.check(lib.dflash_init(), "dflash_init")
+
+    if args.workload != "config4":
+        side_config(lib, args.workload)
+        return
 
     K, W = args.steps, args.warmup
     brk_steps = min(max(K, 1), 16)                 # eager pass with events attached to the kernels
