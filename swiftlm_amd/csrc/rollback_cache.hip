@@ -52,21 +52,20 @@ struct ReplayJob {
     int steps;
 };
 
-// Restores the snapshot and decides whether a replay is needed (RecurrentRollbackCache.swift:95-128).
-int prepare_rollback(dflash_cache* c, int n_accepted, ReplayJob* job, bool* need_replay) {
+// Checks a rollback WITHOUT changing the cache and says whether a tape replay will run
+// (RecurrentRollbackCache.swift:95-128).  Validation is kept apart from the restore so that a call that is
+// going to fail leaves every cache exactly as it was: still armed, tape and snapshot in place.
+int validate_rollback(const dflash_cache* c, int n_accepted, bool* need_replay) {
     *need_replay = false;
     if (!c->has_snapshot) return DFLASH_OK;                       // :96-99, caller clears
-    void* post0 = c->slot[0];
-    void* post1 = c->slot[1];
-    if (c->snap[0]) c->slot[0] = c->snap[0];                      // :108
-    if (c->snap[1]) c->slot[1] = c->snap[1];                      // :109
     if (c->kind != DFLASH_CACHE_TAPE) return DFLASH_OK;           // snapshot-only: :208-214
-    if (!(c->has_tape && c->slot[1])) return DFLASH_OK;           // :112-113
+    const void* restored1 = c->snap[1] ? c->snap[1] : c->slot[1]; // slot 1 as it will be after :108-109
+    if (!(c->has_tape && restored1)) return DFLASH_OK;            // :112-113
     DFLASH_REQUIRE(n_accepted >= 0, "rollback: negative n_accepted");
+    const void* post0 = c->slot[0];
+    const void* post1 = c->slot[1];
     DFLASH_REQUIRE(post1 && post1 != c->snap[1],
                    "rollback: slot 1 still holds the pre-verify buffer; the forward must write a new one");
-    int steps = n_accepted + 1;                                   // :115
-    if (steps > c->T) steps = c->T;                               // slices clamp to the recorded length
     if (c->qkv && c->keep > 0) {
         // The rebuilt window is written into the post-verify conv buffer while snapshot and qkv are read:
         // the three must not share memory (a slice of qkv handed over as the window is a view of it).
@@ -78,9 +77,22 @@ int prepare_rollback(dflash_cache* c, int n_accepted, ReplayJob* job, bool* need
         DFLASH_REQUIRE(post0 && !hits_qkv && !hits_snap,
                        "rollback: slot 0 must be a conv buffer that shares no memory with the snapshot or with qkv");
     }
-    job->c = c; job->post_state = post1; job->post_conv = post0; job->steps = steps;
     *need_replay = true;
     return DFLASH_OK;
+}
+
+// Restores the snapshot (:108-109) of a cache that passed validate_rollback and, when a replay is due, fills in
+// the job.  Cannot fail.
+void restore_snapshot(dflash_cache* c, int n_accepted, bool need_replay, ReplayJob* job) {
+    if (!c->has_snapshot) return;
+    void* post0 = c->slot[0];
+    void* post1 = c->slot[1];
+    if (c->snap[0]) c->slot[0] = c->snap[0];
+    if (c->snap[1]) c->slot[1] = c->snap[1];
+    if (!need_replay) return;
+    int steps = n_accepted + 1;                                   // :115
+    if (steps > c->T) steps = c->T;                               // slices clamp to the recorded length
+    job->c = c; job->post_state = post1; job->post_conv = post0; job->steps = steps;
 }
 
 int finish_rollback(const ReplayJob& j, void* stream) {
@@ -185,8 +197,10 @@ extern "C" int dflash_cache_rollback(dflash_cache_t* c, void* stream, int n_acce
     DFLASH_REQUIRE(is_rollback_kind(c->kind), "cache_rollback: cache kind %d has no rollback", c->kind);
     ReplayJob job;
     bool need = false;
-    int rc = prepare_rollback(c, n_accepted, &job, &need);
-    if (rc == DFLASH_OK && need) rc = replay_jobs(std::vector<ReplayJob>{job}, stream);
+    int rc = validate_rollback(c, n_accepted, &need);
+    if (rc) return rc;                                            // nothing was touched: the cache is still armed
+    restore_snapshot(c, n_accepted, need, &job);
+    if (need) rc = replay_jobs(std::vector<ReplayJob>{job}, stream);
     clear_transients(c);                                          // :130
     return rc;
 }
@@ -211,27 +225,39 @@ extern "C" int dflash_restore_target_cache_after_acceptance(dflash_cache_t* cons
     const bool fully = drafted_tokens > 0 && acceptance_length == drafted_tokens;   // DFlashRuntime.swift:194
     int64_t ns = 0;
     int rc = DFLASH_OK;
-    std::vector<ReplayJob> jobs;
     const auto t0 = std::chrono::steady_clock::now();
-    for (int i = 0; i < n_caches && rc == DFLASH_OK; ++i) {
-        dflash_cache* c = caches[i];
+    // First pass: every handle and every rollback is checked; nothing is changed.  A failure here returns with
+    // all caches as they were (armed, tapes and snapshots in place), so the caller can correct and call again.
+    std::vector<char> need((size_t)n_caches, 0);
+    for (int i = 0; i < n_caches; ++i) {
+        const dflash_cache* c = caches[i];
         DFLASH_REQUIRE(c, "restore_target_cache: null cache handle at %d", i);
+        if (is_rollback_kind(c->kind) && !fully) {
+            bool n = false;
+            rc = validate_rollback(c, acceptance_length, &n);
+            if (rc) return rc;
+            need[(size_t)i] = n;
+        }
+    }
+    // Second pass: restore, collect the replays, fix the offsets.
+    std::vector<ReplayJob> jobs;
+    for (int i = 0; i < n_caches; ++i) {
+        dflash_cache* c = caches[i];
         if (is_rollback_kind(c->kind)) {
             if (fully) { clear_transients(c); continue; }                          // :199-202
             ReplayJob job;
-            bool need = false;
-            rc = prepare_rollback(c, acceptance_length, &job, &need);              // :204
-            if (rc == DFLASH_OK && need) jobs.push_back(job);
+            restore_snapshot(c, acceptance_length, need[(size_t)i] != 0, &job);    // :204
+            if (need[(size_t)i]) jobs.push_back(job);
         } else if (c->kind == DFLASH_CACHE_MAMBA) {
             c->offset = target_len;                                                // :211
         } else if (c->offset > target_len) {                                       // :212-218
             dflash_cache_trim(c, c->offset - target_len);
         }
     }
-    if (rc == DFLASH_OK && !jobs.empty()) rc = replay_jobs(jobs, stream);
+    if (!jobs.empty()) rc = replay_jobs(jobs, stream);
     if (!fully)
         for (int i = 0; i < n_caches; ++i)
-            if (caches[i] && is_rollback_kind(caches[i]->kind)) clear_transients(caches[i]);
+            if (is_rollback_kind(caches[i]->kind)) clear_transients(caches[i]);
     ns = std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now() - t0).count();
     if (replay_ns) *replay_ns = ns;
     return rc;

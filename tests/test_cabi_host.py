@@ -90,7 +90,35 @@ def test_cache_rollback_requires_functional_update():
     # slot 1 still points at the pre-verify buffer: refusing beats corrupting the snapshot
     assert lib.dflash_cache_rollback(c, None, 3) == _lib.INVALID
     assert "pre-verify" in _lib.last_error()
+    # a refused rollback changes nothing: still armed, slots as they were, so the caller can correct and retry
+    assert lib.dflash_cache_is_armed(c)
+    assert lib.dflash_cache_get_slot(c, 0) == 0x1000 and lib.dflash_cache_get_slot(c, 1) == 0x2000
     lib.dflash_cache_destroy(c)
+
+
+def test_restore_validates_every_cache_before_touching_any():
+    """A list whose LAST cache cannot be rolled back (slot 1 still holds the pre-verify buffer), or that holds a
+    null handle, is refused as a whole: the caches before it keep their snapshot, tape, armed flag and offsets."""
+    lib = _lib.load()
+    good, kv, bad = _cache(_lib.CACHE_SNAPSHOT), _cache(_lib.CACHE_KV), _cache(_lib.CACHE_TAPE)
+    lib.dflash_cache_set_slot(good, 1, 0x2000)
+    lib.dflash_cache_arm_rollback(good, 100)
+    lib.dflash_cache_set_slot(good, 1, 0x4000)
+    lib.dflash_cache_set_offset(kv, 116)
+    lib.dflash_cache_set_slot(bad, 0, 0x1000)
+    lib.dflash_cache_set_slot(bad, 1, 0x2000)
+    lib.dflash_cache_arm_rollback(bad, 100)
+    assert lib.dflash_cache_record_tape(bad, 0x10, _lib.F32, 0x20, 0x30, _lib.BF16, 3, None, 2, _lib.F32,
+                                        1, 16, 16, 32, 128, 128, 0) == 0
+    for handles in ([good, kv, bad], [good, kv, C.c_void_p(None)]):
+        arr = (C.c_void_p * 3)(*[h.value for h in handles])
+        rc = lib.dflash_restore_target_cache_after_acceptance(C.cast(arr, _lib.vpp), 3, None, 104, 3, 15, None)
+        assert rc == _lib.INVALID
+        assert lib.dflash_cache_is_armed(good) and lib.dflash_cache_get_slot(good, 1) == 0x4000
+        assert lib.dflash_cache_offset(kv) == 116
+        assert lib.dflash_cache_is_armed(bad) and lib.dflash_cache_get_slot(bad, 1) == 0x2000
+    for h in (good, kv, bad):
+        lib.dflash_cache_destroy(h)
 
 
 def test_snapshot_cache_restores_pointers():
