@@ -400,6 +400,27 @@ int dflash_kv_append(void* stream, void* k_cache, void* v_cache, const void* k_n
                      int offset, const int32_t* offset_dev, int capacity, int32_t* new_len_dev);
 
 /* ------------------------------------------------------------------------
+ * Device-side status word (no counterpart in the reference, whose lengths all live on the host).
+ * Several entries read a length from DEVICE memory (kv_len_dev / cache_len_dev, offset_dev, steps_dev),
+ * so the host cannot check it before the launch.  A value outside the entry's contract never makes a kernel
+ * read or write outside the caller's buffers -- it is clamped, or the write is skipped -- but the result is
+ * then not the one asked for.  To see that it happened, register a device int32 with
+ * dflash_set_status_word(): from then on (for launches enqueued by ANY thread, until it is replaced or
+ * cleared with NULL) the kernels OR the bits below into it, and the caller reads it back whenever it likes,
+ * e.g. together with the accept words.  The library never clears it.
+ *   DFLASH_STATUS_SDPA_LEN      an attention entry found kv_len_dev[b] (or cache_len_dev[b] + M) outside [M, N]
+ *                               and clamped it (a fused append then stored the block at the clamped position)
+ *   DFLASH_STATUS_APPEND_RANGE  dflash_kv_append found rows [offset, offset + M) outside the capacity: nothing
+ *                               was written and new_len_dev was left alone
+ *   DFLASH_STATUS_CONV_STEPS    dflash_rebuild_conv_state found *steps_dev outside [0, T]: rows past the end of
+ *                               the concatenation were left unwritten
+ * ---------------------------------------------------------------------- */
+#define DFLASH_STATUS_SDPA_LEN 1
+#define DFLASH_STATUS_APPEND_RANGE 2
+#define DFLASH_STATUS_CONV_STEPS 4
+int dflash_set_status_word(int32_t* status_dev);
+
+/* ------------------------------------------------------------------------
  * Measurement hook (no counterpart in the reference, whose bench times whole
  * calls from the host: Sources/DFlashKernelBench/main.swift:33-57).  Arms the
  * calling thread so that the NEXT launch of the named kernel carries the two

@@ -17,6 +17,7 @@ OK, UNSUPPORTED, INVALID = 0, 1, 2
 F32, BF16, F16, U8 = 0, 1, 2, 3
 CACHE_TAPE, CACHE_SNAPSHOT, CACHE_MAMBA, CACHE_KV = 0, 1, 2, 3
 MAX_BATCHED_LAYERS = 64
+STATUS_SDPA_LEN, STATUS_APPEND_RANGE, STATUS_CONV_STEPS = 1, 2, 4
 KERNEL_SDPA_PARTIAL, KERNEL_SDPA_COMBINE, KERNEL_GDN_FORWARD, KERNEL_TAPE_REPLAY = 0, 1, 2, 3
 KERNEL_GREEDY_PARTIAL, KERNEL_GDN_PREPARE, KERNEL_EMPTY, KERNEL_GDN_LAYER, KERNEL_GDN_FINISH = 4, 5, 6, 7, 8
 
@@ -50,6 +51,7 @@ SIGNATURES = {
     "dflash_greedy_accept_commit": (i32, [vp, vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, sz]),
     "dflash_rebuild_conv_state": (i32, [vp, vp, vp, vp] + [i32] * 6 + [vp]),
     "dflash_kv_append": (i32, [vp, vp, vp, vp, vp] + [i32] * 5 + [i64, i64, i32, vp, i32, vp]),
+    "dflash_set_status_word": (i32, [vp]),
     "dflash_profile_next_launch": (i32, [i32, vp, vp]),
     "dflash_profile_empty_launch": (i32, [vp, i32, i32, i32, i32, i32]),
     "dflash_cache_create": (vp, [i32, i32]),

@@ -44,6 +44,7 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
     } while (0)
 
 int ensure_init();           // per-device one-time setup; 0 or negative hip error
+int32_t* status_word();      // the device int32 registered with dflash_set_status_word(), or null
 int num_compute_units();     // of the current device (cached)
 
 // Per-device setup of the kernel files, run once per device by ensure_init() under its mutex with that

@@ -9,6 +9,8 @@
 
 #include <type_traits>
 
+#include <atomic>
+
 #include "dflash_common.h"
 
 namespace dflash {
@@ -224,8 +226,11 @@ __global__ __launch_bounds__(kArgmaxThreads) void greedy_finish_kernel(GreedyArg
 
 // out[b, j, :] = concat(snapshot [B,keep,C], qkv [B,T,C])[b, s + j, :], 16-byte pieces.
 __global__ __launch_bounds__(256) void rebuild_conv_kernel(const uint4* snap, const uint4* qkv, uint4* out, int keep,
-                                                           int T, int C16, int steps, const int32_t* steps_dev) {
+                                                           int T, int C16, int steps, const int32_t* steps_dev,
+                                                           int32_t* status) {
     int s = steps_dev ? *steps_dev : steps;
+    if (status && (s < 0 || s > T) && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
+        atomicOr(status, DFLASH_STATUS_CONV_STEPS);
     s = s < 0 ? 0 : s;
     const int b = blockIdx.z, j = blockIdx.y;
     const int src = s + j;
@@ -243,9 +248,12 @@ __global__ __launch_bounds__(256) void rebuild_conv_kernel(const uint4* snap, co
 __global__ __launch_bounds__(256) void kv_append_kernel(uint4* k_cache, uint4* v_cache, const uint4* k_new,
                                                         const uint4* v_new, int Hk, int M, int D16, long batch_stride16,
                                                         long head_stride16, int offset, const int32_t* offset_dev,
-                                                        int capacity, int32_t* new_len_dev) {
+                                                        int capacity, int32_t* new_len_dev, int32_t* status) {
     int off = offset_dev ? *offset_dev : offset;
-    if (off < 0 || off + M > capacity) return;   // never write outside the cache
+    if (off < 0 || off + M > capacity) {          // never write outside the cache
+        if (status && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) atomicOr(status, DFLASH_STATUS_APPEND_RANGE);
+        return;
+    }
     if (new_len_dev && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *new_len_dev = off + M;
     const int bh = blockIdx.y;
     const int b = bh / Hk, hk = bh % Hk;
@@ -261,6 +269,13 @@ __global__ __launch_bounds__(256) void kv_append_kernel(uint4* k_cache, uint4* v
 }  // namespace dflash
 
 using namespace dflash;
+
+static std::atomic<int32_t*> g_status_word{nullptr};
+int32_t* dflash::status_word() { return g_status_word.load(std::memory_order_acquire); }
+extern "C" int dflash_set_status_word(int32_t* status_dev) {
+    g_status_word.store(status_dev, std::memory_order_release);
+    return DFLASH_OK;
+}
 
 extern "C" int dflash_version(void) { return 100; }
 extern "C" const char* dflash_last_error(void) { return g_err; }
@@ -392,7 +407,7 @@ extern "C" int dflash_rebuild_conv_state(void* stream, const void* snapshot_conv
     const int C16 = (int)(((long)C * elem_bytes) / 16);
     dim3 grid((C16 + 255) / 256, keep, B);
     hipLaunchKernelGGL(rebuild_conv_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const uint4*)snapshot_conv,
-                       (const uint4*)tape_qkv, (uint4*)out, keep, T, C16, accepted_steps, steps_dev);
+                       (const uint4*)tape_qkv, (uint4*)out, keep, T, C16, accepted_steps, steps_dev, status_word());
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
 }
@@ -416,7 +431,7 @@ extern "C" int dflash_kv_append(void* stream, void* k_cache, void* v_cache, cons
     dim3 grid((M * D16 + 255) / 256, B * Hk);
     hipLaunchKernelGGL(kv_append_kernel, grid, dim3(256), 0, (hipStream_t)stream, (uint4*)k_cache, (uint4*)v_cache,
                        (const uint4*)k_new, (const uint4*)v_new, Hk, M, D16, (long)(kv_batch_stride * elem_bytes / 16),
-                       (long)(kv_head_stride * elem_bytes / 16), offset, offset_dev, capacity, new_len_dev);
+                       (long)(kv_head_stride * elem_bytes / 16), offset, offset_dev, capacity, new_len_dev, status_word());
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
 }

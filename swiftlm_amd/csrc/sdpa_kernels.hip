@@ -98,6 +98,7 @@ struct SdpaArgs {
     // kv_head_stride the head pitch inside a page.
     const int32_t* page_table;
     int page_shift, table_stride, num_pages;
+    int32_t* status;         // device status word (dflash_set_status_word), or null
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -223,7 +224,8 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
     asm volatile("" ::"s"(A.q), "s"(A.k), "s"(A.v), "s"(A.k_new), "s"(A.v_new), "s"(A.k_cache), "s"(A.v_cache), "s"(A.part_o),
                  "s"(A.part_m), "s"(A.part_l), "s"(A.kv_len_dev), "s"(A.mask), "s"(A.kv_batch_stride), "s"(A.kv_head_stride));
     asm volatile("" ::"s"(A.scale_log2), "s"(A.Hq), "s"(A.Hk), "s"(A.G), "s"(A.N), "s"(A.S), "s"(A.groups_per_kv),
-                 "s"(A.rows_total), "s"(A.len_bias), "s"(A.page_table), "s"(A.page_shift), "s"(A.table_stride), "s"(A.num_pages));
+                 "s"(A.rows_total), "s"(A.len_bias), "s"(A.page_table), "s"(A.page_shift), "s"(A.table_stride), "s"(A.num_pages),
+                 "s"(A.status));
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -292,6 +294,7 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
     }
     asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(len_raw));
     int Nb = A.kv_len_dev ? len_raw + A.len_bias : A.N;
+    if (A.status && (Nb < kM || Nb > A.N) && split == 0 && blockIdx.y == 0 && tid == 0) atomicOr(A.status, DFLASH_STATUS_SDPA_LEN);
     Nb = Nb < kM ? kM : (Nb > A.N ? A.N : Nb);
     const int nt = (Nb + kBN - 1) / kBN;
     // Tiles are dealt round-robin: split s takes tiles s, s + S, s + 2S, ...  At any moment the workgroups of a KV
@@ -1036,6 +1039,7 @@ static int sdpa_common(void* stream, const void* q, const void* k, const void* v
     A.page_shift = page_shift;
     A.table_stride = paged ? paged->table_stride : 0;
     A.num_pages = paged ? paged->num_pages : 0;
+    A.status = status_word();
     CombineArgs C;
     C.part_o = A.part_o; C.part_m = A.part_m; C.part_l = A.part_l;
     C.out = (uint16_t*)out; C.lse = lse; C.S = S;

@@ -378,3 +378,56 @@ def test_verify_stack_paged_equals_dense(gpu_lib):
         for ld, lp in zip(dense.gdn, paged.gdn):
             assert torch.equal(ld["state"][dense.phase], lp["state"][paged.phase])
 
+
+
+def test_device_status_word_reports_out_of_contract_device_lengths(gpu_lib):
+    """Lengths read from device memory cannot be checked by the host.  Out of contract they are clamped (or the
+    write is skipped) and the registered status word receives a bit per kind; in contract it stays 0."""
+    from swiftlm_amd import DFlashKernels as K, _lib
+    from swiftlm_amd.dflash_kernels import _ptr, _stream
+
+    lib = _lib.load()
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    assert lib.dflash_set_status_word(_ptr(status)) == 0
+    try:
+        B, Hq, Hk, D, cap = 1, 4, 2, 128, 96
+        g = torch.Generator(device="cuda").manual_seed(3)
+        q = torch.randn(B, Hq, 16, D, generator=g, device="cuda").bfloat16()
+        kc = torch.randn(B, Hk, cap, D, generator=g, device="cuda").bfloat16()
+        vc = torch.randn(B, Hk, cap, D, generator=g, device="cuda").bfloat16()
+        kn = torch.randn(B, Hk, 16, D, generator=g, device="cuda").bfloat16()
+        vn = torch.randn(B, Hk, 16, D, generator=g, device="cuda").bfloat16()
+        # in contract: 40 cached rows + 16 <= n_keys = 64
+        good = torch.tensor([40], dtype=torch.int32, device="cuda")
+        K.batched_sdpa_2pass_append(q, kc.clone(), vc.clone(), kn, vn, D ** -0.5, 64, cache_len=good)
+        torch.cuda.synchronize()
+        assert int(status) == 0
+        # out of contract: 60 cached rows + 16 > 64 -> clamped to 64 keys, flagged; rows beyond the bound stay untouched
+        bad = torch.tensor([60], dtype=torch.int32, device="cuda")
+        kc2, vc2 = kc.clone(), vc.clone()
+        out = K.batched_sdpa_2pass_append(q, kc2, vc2, kn, vn, D ** -0.5, 64, cache_len=bad)
+        torch.cuda.synchronize()
+        assert int(status) == _lib.STATUS_SDPA_LEN
+        assert torch.isfinite(out.float()).all()
+        assert torch.equal(kc2[:, :, 64:], kc[:, :, 64:]) and torch.equal(vc2[:, :, 64:], vc[:, :, 64:])
+        # kv_append past the capacity: nothing written, flagged
+        status.zero_()
+        off = torch.tensor([cap - 8], dtype=torch.int32, device="cuda")
+        kc3 = kc.clone()
+        rc = lib.dflash_kv_append(_stream(), _ptr(kc3), _ptr(vc.clone()), _ptr(kn), _ptr(vn), B, Hk, 16, D, 2,
+                                  kc3.stride(0), kc3.stride(1), 0, _ptr(off), cap, None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert int(status) == _lib.STATUS_APPEND_RANGE and torch.equal(kc3, kc)
+        # conv rebuild with a step count beyond the tape
+        status.zero_()
+        keep, T, C = 3, 4, 64
+        snap = torch.randn(B, keep, C, generator=g, device="cuda").bfloat16()
+        qkv = torch.randn(B, T, C, generator=g, device="cuda").bfloat16()
+        dst = torch.zeros(B, keep, C, dtype=torch.bfloat16, device="cuda")
+        steps = torch.tensor([T + 3], dtype=torch.int32, device="cuda")
+        assert lib.dflash_rebuild_conv_state(_stream(), _ptr(snap), _ptr(qkv), _ptr(dst), B, keep, T, C, 2, 0, _ptr(steps)) == 0
+        torch.cuda.synchronize()
+        assert int(status) == _lib.STATUS_CONV_STEPS
+    finally:
+        lib.dflash_set_status_word(None)
