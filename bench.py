@@ -312,6 +312,32 @@ def aux_kernels(lib, cfg, reps=48):
 
     out["gdn_layer"] = aux_gdn_layer(lib, cfg)
 
+    # The same forward with the state kept in the input type (what the reference's Metal kernel emits for bf16 q,
+    # DFlashKernels.swift:340,364: re-rounded after every step, so it cannot take the chunked form and runs the
+    # serial kernel) next to the fp32-state forward the benchmark step uses.
+    qs = [(torch.nn.functional.normalize(torch.randn(B, T, Hk, Dk, generator=g, device=dev), dim=-1).to(bf),
+           torch.nn.functional.normalize(torch.randn(B, T, Hk, Dk, generator=g, device=dev), dim=-1).to(bf),
+           torch.randn(B, T, Hv, Dv, generator=g, device=dev).to(bf),
+           torch.rand(B, T, Hv, generator=g, device=dev).to(bf), torch.rand(B, T, Hv, generator=g, device=dev).to(bf),
+           0.1 * torch.randn(B, Hv, Dv, Dk, generator=g, device=dev)) for _ in range(reps)]
+    for label, cast in (("gdn_forward_fp32_state", lambda s: s), ("gdn_forward_bf16_state", lambda s: s.to(bf))):
+        sets2 = [(q_, k_, v_, g_, b_, cast(s_)) for q_, k_, v_, g_, b_, s_ in qs]
+        for a_ in sets2[:4]:
+            K.gated_delta_kernel_with_tape(*a_)
+        ev = HipEvents()
+        for a_ in sets2:
+            e0, e1 = ev.pair()
+            _lib.check(lib.dflash_profile_next_launch(_lib.KERNEL_GDN_FORWARD, e0, e1), "profile_next_launch")
+            K.gated_delta_kernel_with_tape(*a_)
+        torch.cuda.synchronize()
+        us = float(np.median(ev.durations_us()))
+        sb = 4 if label.endswith("fp32_state") else 2
+        nbytes = 2 * Hv * Dv * Dk * sb + (2 * T * Hk * Dk + T * Hv * Dv + 2 * T * Hv) * 2 + T * Hv * Dv * 2 + T * Hv * Dv * 4
+        out[label] = {"us": round(us, 2), "algorithmic_bytes": nbytes, "gbs": round(nbytes / us / 1e3, 1),
+                      "kernel": "chunked (MFMA)" if sb == 4 else "serial (state re-rounded per step)"}
+        ev.destroy()
+    del qs
+
     V = 151936
     logits = [torch.randn(T, V, generator=g, device=dev).to(bf) for _ in range(reps)]      # 48 x 4.9 MB
     mask = R.build_suppress_token_mask(V, [1, 2, 3])

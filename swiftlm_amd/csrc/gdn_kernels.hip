@@ -615,12 +615,14 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
     // Every kernel argument is asked for here, in one burst of scalar loads.  Left alone the compiler fetches
     // them where they are first used, in three or four dependent rounds, and each round that touches a new
     // cache line of the argument block is a trip to memory on the way to the first global load.
-    asm volatile("" ::"s"(A.q), "s"(A.k), "s"(A.v), "s"(A.g), "s"(A.beta), "s"(A.mask), "s"(A.state_in), "s"(A.state_out),
-                 "s"(A.y), "s"(A.tape), "s"(A.in_dtype), "s"(A.mask_dtype), "s"(A.T), "s"(A.Hk), "s"(A.Hv), "s"(A.Dv));
     if constexpr (FUSED)
-        asm volatile("" ::"s"(P.x), "s"(P.conv_in), "s"(P.weight), "s"(P.a), "s"(P.b), "s"(P.a_log), "s"(P.dt_bias),
-                     "s"(P.q_out), "s"(P.k_out), "s"(P.v_out), "s"(P.g_out), "s"(P.beta_out), "s"(P.conv_out),
+        asm volatile("" ::"s"(A.state_in), "s"(A.state_out), "s"(A.y), "s"(A.tape), "s"(A.in_dtype), "s"(A.T), "s"(A.Hk),
+                     "s"(A.Hv), "s"(A.Dv), "s"(P.x), "s"(P.conv_in), "s"(P.weight), "s"(P.a), "s"(P.b), "s"(P.a_log),
+                     "s"(P.dt_bias), "s"(P.q_out), "s"(P.k_out), "s"(P.v_out), "s"(P.g_out), "s"(P.beta_out), "s"(P.conv_out),
                      "s"(P.q_scale), "s"(P.k_scale), "s"(P.eps), "s"(P.C));
+    else
+        asm volatile("" ::"s"(A.q), "s"(A.k), "s"(A.v), "s"(A.g), "s"(A.beta), "s"(A.mask), "s"(A.state_in), "s"(A.state_out),
+                     "s"(A.y), "s"(A.tape), "s"(A.in_dtype), "s"(A.mask_dtype), "s"(A.T), "s"(A.Hk), "s"(A.Hv), "s"(A.Dv));
     constexpr int E = DK / 64;             // channels per lane in the state-update product (16 lanes x E x 4 waves = DK)
     static_assert(DK % 64 == 0, "chunked gated delta needs Dk to be a multiple of 64");
 
