@@ -764,7 +764,10 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 const int r = r0 + u * RPP + rsub;
-                if (r < rows) *reinterpret_cast<u32x4_t*>(dst + (size_t)r * D) = o[u];
+                // Written through (system scope): the 16.8 MB of partial rows then drain while other workgroups still
+                // compute, instead of sitting dirty in the L2s until the end-of-launch flush (-0.7 us per launch).
+                if (r < rows)
+                    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"((uint64_t)(dst + (size_t)r * D)), "v"(o[u]) : "memory");
             }
         }
     }
