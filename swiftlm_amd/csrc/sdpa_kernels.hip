@@ -766,8 +766,10 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
                 const int r = r0 + u * RPP + rsub;
                 // Written through (system scope): the 16.8 MB of partial rows then drain while other workgroups still
                 // compute, instead of sitting dirty in the L2s until the end-of-launch flush (-0.7 us per launch).
+                // (The s_nop is the wait state the hardware needs between a store of more than 64 bits and a VALU write
+                //  of the registers that hold its data; the compiler inserts it for its own stores, not for assembly.)
                 if (r < rows)
-                    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"((uint64_t)(dst + (size_t)r * D)), "v"(o[u]) : "memory");
+                    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"((uint64_t)(dst + (size_t)r * D)), "v"(o[u]) : "memory");
             }
         }
     }
