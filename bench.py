@@ -6,7 +6,7 @@ A "step" is one verify step of the hybrid stack of the headline benchmark config
 context, accepted length ~ Geometric(0.25) clipped to [1, 16].  Per step: 36
 GatedDelta forwards with tape, 12 KV appends + block-causal SDPAs, the accept kernel
 and one batched tape replay, all resident in HBM, enqueued through the C ABI.
-Steps are captured in HIP graphs (two steps per graph, the state buffers ping-pong)
+Steps are captured in HIP graphs (eight steps per graph by default, the state buffers ping-pong)
 unless --no-graph is given.
 
 Prints ONE JSON line.  `value` is microseconds per layer (step time / 48).  The
@@ -502,6 +502,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--no-graph", action="store_true", help="enqueue every step from the host instead of replaying graphs")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--steps-per-graph", type=int, default=8, help="verify steps captured per HIP graph (even)")
     ap.add_argument("--context", type=int, default=32768)
     ap.add_argument("--aux", action="store_true",
                     help="also time the kernels next to the measured path (pre-ops, greedy tokens) and report them "
@@ -536,8 +537,9 @@ def main():
     K, W = args.steps, args.warmup
     brk_steps = min(max(K, 1), 16)                 # eager pass with events attached to the kernels
     total = 2 + W + K + brk_steps + 2              # + the two checked steps after the timed region
+    G = max(2, args.steps_per_graph & ~1)
     cfg = StackConfig(context=args.context, max_steps=total + 2, page_size=args.page_size)
-    stack = HybridVerifyStack(cfg, seed=0)
+    stack = HybridVerifyStack(cfg, seed=0, n_slots=G)
     T = cfg.block
     commits = draw_commit_counts(total, T)
     # token ids of every step, staged on the device once
@@ -552,27 +554,15 @@ def main():
         if cc - 1 < T - 1:
             p[cc - 1] = row[cc] + 1                # first mismatch -> acceptance length cc - 1
         ids[s], post[s] = row, p
-    # [step, ids | posterior, T]: one device-to-device copy hands a step its token ids (what the drafter and the
-    # target's argmax would leave on the device), two consecutive steps' worth when a graph holds two steps
+    # [step, ids | posterior, T]: one device-to-device copy hands the steps of a graph their token ids (what the
+    # drafter and the target's argmax would leave on the device)
     staged_d = torch.stack([ids, post], dim=1).cuda()
     step_no = [0]
 
-    def stage(phase):
-        s = step_no[0]
-        stack.accept_inputs[phase].copy_(staged_d[s], non_blocking=True)
-        step_no[0] += 1
-
-    def stage_pair(phase):
-        s = step_no[0]
-        if phase == 0:
-            stack.accept_inputs.copy_(staged_d[s:s + 2], non_blocking=True)
-        else:
-            stage(phase); stage(1 - phase)
-            return
-        step_no[0] += 2
-
     def eager_step(before_launch=None):
-        stage(stack.phase)
+        s = step_no[0]
+        stack.accept_inputs[stack.phase].copy_(staged_d[s], non_blocking=True)
+        step_no[0] += 1
         stack.enqueue_step(before_launch=before_launch)
 
     # two eager steps first: loads code objects, sets LDS attributes (not legal during capture)
@@ -580,35 +570,56 @@ def main():
     torch.cuda.synchronize()
     assert int(stack.offset) == cfg.context + commits[0] + commits[1], "device-side commit bookkeeping is off"
 
-    graphs = None
-    if not args.no_graph:
-        # one graph per starting phase of the ping-pong state buffers, two steps each
-        graphs = {}
-        side = torch.cuda.Stream()
-        for ph in (0, 1):
+    def chunks(n):
+        """n steps as graph replays of G steps, one of the even remainder, and a last eager step if n is odd."""
+        out = [G] * (n // G)
+        if (n % G) & ~1:
+            out.append((n % G) & ~1)
+        if n & 1:
+            out.append(1)
+        return out
+
+    # one graph per (starting phase of the ping-pong state buffers, number of steps), captured when first needed and
+    # always outside the timed region; every graph holds an even number of steps, so the phase only changes with an
+    # odd eager step
+    graphs = None if args.no_graph else {}
+    cap = torch.cuda.Stream()
+
+    def graph_for(ph, m):
+        if (ph, m) not in graphs:
+            keep = stack.phase
             stack.phase = ph
-            side.wait_stream(torch.cuda.current_stream())
+            cap.wait_stream(torch.cuda.current_stream())
             g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g, stream=side):
-                stack.enqueue_step()
-                stack.enqueue_step()
-            torch.cuda.current_stream().wait_stream(side)
-            graphs[ph] = g
-        stack.phase = 0
-        torch.cuda.synchronize()
+            with torch.cuda.graph(g, stream=cap):
+                for i in range(m):
+                    stack.enqueue_step(slot=i)
+            torch.cuda.current_stream().wait_stream(cap)
+            stack.phase = keep
+            graphs[(ph, m)] = g
+        return graphs[(ph, m)]
+
+    def precapture(n_steps):
+        ph = stack.phase
+        for m in chunks(n_steps):
+            if m == 1:
+                ph = 1 - ph
+            else:
+                graph_for(ph, m)
 
     def run(n_steps):
-        for _ in range(n_steps // 2):
-            if graphs is not None:
-                ph = stack.phase
-                stage_pair(ph)
-                graphs[ph].replay()
-            else:
-                eager_step(); eager_step()
-        if n_steps & 1:
-            eager_step()
+        for m in (chunks(n_steps) if graphs is not None else [1] * n_steps):
+            if m == 1:
+                eager_step()
+                continue
+            s = step_no[0]
+            stack.accept_inputs[:m].copy_(staged_d[s:s + m], non_blocking=True)
+            step_no[0] += m
+            graph_for(stack.phase, m).replay()
 
     run(W)
+    if graphs is not None:
+        precapture(K)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     run(K)
@@ -695,7 +706,7 @@ def main():
                          "16-token block, L=%d, accepted n ~ Geometric(0.25) in [1,16]; GatedDelta Hk=16 Hv=32 dk=dv=128 "
                          "fp32 state; attention Hq=16 Hkv=2 D=256 bf16") % cfg.context,
             "layers": cfg.n_layers, "block": T, "context": cfg.context,
-            "launch": "eager" if graphs is None else "hip-graph, 2 steps per graph",
+            "launch": "eager" if graphs is None else "hip-graph, %d steps per graph" % G,
             "kv_layout": "dense" if not cfg.page_size else "paged, %d-key pages" % cfg.page_size,
         },
         "verified": True,
@@ -708,7 +719,7 @@ def main():
         "step_frac_of_hbm_peak": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "launch_floor": {
             "us_per_step": round(floor_us, 1), "launches_per_step": n_launches, "us_per_launch": round(floor_us / n_launches, 2),
-            "how": "HIP graph of empty kernels with every step kernel's grid, block and LDS size, two steps per graph, 50 replays",
+            "how": "HIP graph of empty kernels with every step kernel's grid, block and LDS size, in one chain, two steps per graph, 50 replays",
         },
         "step_minus_floor_ms": round(ms_per_step - floor_us * 1e-3, 4),
         "step_frac_of_hbm_peak_above_floor": round(step_bytes / ((ms_per_step - floor_us * 1e-3) * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),

@@ -64,7 +64,7 @@ def _p(t: Optional[torch.Tensor]):
 class HybridVerifyStack:
     """Buffers plus the enqueue routine of one verify step."""
 
-    def __init__(self, cfg: StackConfig, seed: int = 0, device: str = "cuda"):
+    def __init__(self, cfg: StackConfig, seed: int = 0, device: str = "cuda", n_slots: int = 2):
         self.cfg = cfg
         self.lib = _lib.load()
         self.fuse_accept = True      # acceptance decided inside the batched replay launch (one launch fewer per step)
@@ -125,9 +125,10 @@ class HybridVerifyStack:
         self.accept = torch.zeros(4, dtype=torch.int32, device=device)
         # acceptance inputs of the step being enqueued, one pair per ping-pong phase
         # (one block [phase, ids | posterior, T], so that a caller can hand over both phases with a single copy)
-        self.accept_inputs = torch.zeros(2, 2, T, dtype=torch.int32, device=device)
-        self.verify_ids = [self.accept_inputs[ph, 0] for ph in range(2)]
-        self.posterior = [self.accept_inputs[ph, 1] for ph in range(2)]
+        # (n_slots > 2: a graph that holds more than two steps gives every step its own slot)
+        self.accept_inputs = torch.zeros(max(n_slots, 2), 2, T, dtype=torch.int32, device=device)
+        self.verify_ids = [self.accept_inputs[i, 0] for i in range(self.accept_inputs.shape[0])]
+        self.posterior = [self.accept_inputs[i, 1] for i in range(self.accept_inputs.shape[0])]
         self.phase = 0               # which state buffer holds the pre-verify state
         # host pointer tables for the batched replay, one per phase
         self._tables = []
@@ -139,13 +140,15 @@ class HybridVerifyStack:
                 sout=mk([l["state"][1 - ph] for l in self.gdn])))
 
     # -- one step ------------------------------------------------------------------
-    def enqueue_step(self, stream: Optional[int] = None, before_launch=None) -> None:
+    def enqueue_step(self, stream: Optional[int] = None, before_launch=None, slot: Optional[int] = None) -> None:
         """Enqueue one verify step.  ``before_launch(name)`` is called ahead of each kernel-launching
-        C call with name in {"gdn_forward", "sdpa", "tape_replay"} (used to arm timing brackets)."""
+        C call with name in {"gdn_forward", "sdpa", "tape_replay"} (used to arm timing brackets).
+        ``slot``: which row of ``accept_inputs`` holds this step's token ids (default: the phase)."""
         cfg, lib, T = self.cfg, self.lib, self.cfg.block
         note = before_launch or (lambda name: None)
         st = C.c_void_p(torch.cuda.current_stream().cuda_stream if stream is None else stream)
         ph = self.phase
+        slot = ph if slot is None else slot
         gi = ai = 0
         for kind in cfg.kinds():
             if kind == "gdn":
@@ -181,14 +184,14 @@ class HybridVerifyStack:
             tb = self._tables[ph]
             note("tape_replay")
             rc = lib.dflash_accept_commit_replay_batched(
-                st, _p(self.verify_ids[ph]), _p(self.posterior[ph]), T, _p(self.offset), _p(self.accept),
+                st, _p(self.verify_ids[slot]), _p(self.posterior[slot]), T, _p(self.offset), _p(self.accept),
                 len(self.gdn), cast(tb["tape"]), _lib.F32, cast(tb["k"]), cast(tb["g"]), _lib.BF16, 3,
                 cast(tb["sin"]), cast(tb["sout"]), _lib.F32, 1, 1, T, cfg.Hk, cfg.Hv, cfg.Dk, cfg.Dv)
             _lib.check(rc, "accept_commit_replay_batched")
             self.phase = 1 - ph
             return
         # accept: commit count -> accept[1]; offset += commit count
-        rc = lib.dflash_accept_commit(st, _p(self.verify_ids[ph]), _p(self.posterior[ph]), T, _p(self.offset),
+        rc = lib.dflash_accept_commit(st, _p(self.verify_ids[slot]), _p(self.posterior[slot]), T, _p(self.offset),
                                       _p(self.accept))
         _lib.check(rc, "accept_commit")
         # rollback: every GatedDelta layer in one launch, step count read on the device
