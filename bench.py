@@ -361,7 +361,8 @@ def aux_kernels(lib, cfg, reps=48):
 def aux_gdn_layer(lib, cfg, n_layers=36, reps=30):
     """A GatedDelta layer's body between its projections (conv + SiLU, q/k norm, gates, recurrence with tape,
     gated norm) at the benchmark's shapes, as the three calls prepare -> forward -> finish and as the one call
-    dflash_gdn_layer (pre-ops inside the forward kernel): `n_layers` layers with their own inputs and states
+    dflash_gdn_layer (pre-ops inside the forward kernel's load phase, gated norm by the last workgroup of each
+    head; also with the gated norm as a second launch): `n_layers` layers with their own inputs and states
     captured into one HIP graph each way, microseconds per layer by the host clock around `reps` replays, and
     the kernels' own durations by events on an eager pass."""
     import torch
@@ -382,18 +383,21 @@ def aux_gdn_layer(lib, cfg, n_layers=36, reps=30):
         y, s1, tape = K.gated_delta_kernel_with_tape(q, k, v, gg, beta, l["s0"])
         return K.gdn_finish(y, l["z"], l["nw"], 1e-6, "silu"), s1, tape, k, gg, conv
 
-    def one(l):
+    def one(l, one_launch=True):
         r = K.gdn_layer(l["x"], l["st"], l["w"], l["a"], l["b"], l["a_log"], l["dt_bias"], l["s0"], Hk, Hv, Dk, Dv, **sc,
-                        gate=l["z"], norm_weight=l["nw"], norm_eps=1e-6, gate_kind="silu")
+                        gate=l["z"], norm_weight=l["nw"], norm_eps=1e-6, gate_kind="silu", one_launch=one_launch)
         return r["out"], r["state"], r["tape"], r["k"], r["g"], r["conv_state"]
+
+    def two(l):              # the one call with the gated norm as a second launch
+        return one(l, False)
 
     res = {"shape": "B=1 T=%d Hk=%d Hv=%d Dk=%d Dv=%d K=%d bf16, fp32 state, %d layers per graph" % (T, Hk, Hv, Dk, Dv, Kc, n_layers)}
     same = True
     for l in layers[:3]:
-        same = same and all(torch.equal(a, b) for a, b in zip(three(l), one(l)))
+        same = same and all(torch.equal(a, b) and torch.equal(a, c) for a, b, c in zip(three(l), one(l), two(l)))
     res["one_call_equals_three_calls_bitwise"] = bool(same)
     side = torch.cuda.Stream()
-    for name, fn, launches in (("three_calls", three, 3), ("one_call", one, 2)):
+    for name, fn, launches in (("three_calls", three, 3), ("one_call_norm_as_second_launch", two, 2), ("one_call", one, 1)):
         torch.cuda.synchronize()
         side.wait_stream(torch.cuda.current_stream())
         graph = torch.cuda.CUDAGraph()

@@ -162,10 +162,10 @@ int dflash_gdn_finish(void* stream, const void* y, const void* gate, const void*
  * (Sources/SwiftLM/KimiLinearDFlash.swift:351-378: short conv + SiLU, q/k normalisation, gates,
  * the recurrence through DFlashKernelProvider.gatedDeltaKernelWithTape, oNorm(out) * act(gate)).
  * Equivalent to dflash_gdn_prepare -> dflash_gated_delta_tape -> dflash_gdn_finish, bit for bit,
- * in two launches instead of three: the pre-ops run inside the forward kernel's load phase, so
- * q, k, v, g and beta never travel through memory; the gated norm stays a launch of its own
- * because it normalises over the Dv rows of a head, which the forward spreads over several
- * workgroups.
+ * in one launch instead of three: the pre-ops run inside the forward kernel's load phase, so
+ * q, k, v, g and beta never travel through memory, and the gated norm -- which normalises over
+ * the Dv rows of a head, spread by the forward over Dv/16 workgroups -- is done by whichever of
+ * those workgroups finishes last (each counts itself in `arrivals`; none waits for another).
  *   inputs    mixed_qkv, conv_state_in (or NULL), conv_weight, a_logits [B,T,Hv], b_logits,
  *             A_log, dt_bias [Hv], q_scale, k_scale, norm_eps as for dflash_gdn_prepare;
  *             state_in [B,Hv,Dv,Dk] float32
@@ -175,7 +175,12 @@ int dflash_gdn_finish(void* stream, const void* y, const void* gate, const void*
  *             (RecurrentRollbackCache.swift:75-85), NULL to skip;
  *             q_out, v_out, beta_out: optional copies of the other pre-op results, NULL to skip
  *   gate      NULL: stop after the recurrence.  Otherwise gate [B,T,Hv,Dv], out_norm_weight [Dv],
- *             out_norm_eps, gate_kind and out [B,T,Hv,Dv] as for dflash_gdn_finish.
+ *             out_norm_eps, gate_kind and out [B,T,Hv,Dv] as for dflash_gdn_finish (out must not
+ *             alias y_out).
+ *   arrivals  device int32 [B*Hv], all zero before the call; the call leaves it all zero, so one
+ *             array zeroed once serves every later call that does not overlap with another one
+ *             using the same array (calls on one stream never overlap).  NULL, or Dv > 256: the
+ *             gated norm runs as a second launch, as dflash_gdn_finish.
  * Covers the verify block: float32 state, one decay per head and step, no step mask, K == 4,
  * T <= 16, Dk in {64, 128, 256}, Dv a multiple of 16.  Anything else returns
  * DFLASH_UNSUPPORTED and the caller issues the three calls.
@@ -188,7 +193,7 @@ int dflash_gdn_layer(void* stream,
                      const void* state_in, void* state_out,
                      void* k_out, void* g_out, float* tape_out, void* conv_state_out, void* y_out,
                      const void* gate, const void* out_norm_weight, float out_norm_eps, int gate_kind,
-                     void* out,
+                     void* out, int32_t* arrivals,
                      void* q_out, void* v_out, void* beta_out,
                      int B, int T, int Hk, int Hv, int Dk, int Dv, int K);
 

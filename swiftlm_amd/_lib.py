@@ -34,7 +34,7 @@ SIGNATURES = {
     "dflash_gated_delta_tape": (i32, [vp, vp, vp, vp, vp, i32, vp, i32, vp, vp, i32, vp, vp, vp, i32] + [i32] * 6),
     "dflash_gdn_prepare": (i32, [vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, f32, f32, f32, vp, vp, vp, vp, vp, vp] + [i32] * 7),
     "dflash_gdn_finish": (i32, [vp, vp, vp, vp, vp, i32, f32, i32, i32, i32, i32, i32]),
-    "dflash_gdn_layer": (i32, [vp] * 8 + [i32, f32, f32, f32] + [vp] * 9 + [f32, i32] + [vp] * 4 + [i32] * 7),
+    "dflash_gdn_layer": (i32, [vp] * 8 + [i32, f32, f32, f32] + [vp] * 9 + [f32, i32] + [vp] * 5 + [i32] * 7),
     "dflash_sdpa_workspace_bytes": (sz, [i32] * 6),
     "dflash_sdpa_block_causal": (i32, [vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp, vp, sz]),
     "dflash_sdpa_block_causal_static": (i32, [vp, vp, vp, vp, vp, vp, i32, f32] + [i32] * 6 + [i64, i64, vp]),

@@ -146,6 +146,16 @@ __device__ __forceinline__ float gdn_norm_scale(float sumsq, int dim, float eps,
     return scale * rsqrtf(sumsq / (float)dim + eps);
 }
 
+// The layer's gated output norm, out = rmsNorm(y; weight, eps) * act(gate) (KimiLinearDFlash.swift:377-378), is
+// computed by the post-op kernel and by the one-launch layer kernel; both sum the squares of a row the same way --
+// 16 consecutive channels by group_sum<16>, then those sums added one after the other from channel 0 up, starting
+// from 0 -- and share these two expressions, so that they agree bit for bit.
+__device__ __forceinline__ float gdn_rms_inv(float sumsq, int dim, float eps) { return rsqrtf(sumsq / (float)dim + eps); }
+__device__ __forceinline__ float gdn_gated_out(float y, float inv, float w, float z, bool silu_gate) {
+    const float act = silu_gate ? z * sigmoid_f(z) : sigmoid_f(z);
+    return y * inv * w * act;
+}
+
 // mask element of run-time type -> "this step runs"
 __device__ __forceinline__ bool mask_on(const void* mask, int mask_dtype, int idx) {
     float m;

@@ -41,6 +41,39 @@ __device__ __forceinline__ void store1_rt(void* base, int dtype, size_t idx, flo
     }
 }
 
+// The same store and its load at agent scope: written through to, and read from, the level of the memory system
+// that every workgroup of the launch shares (each XCD has an L2 of its own).  Data handed from one workgroup to
+// another inside a launch goes this way; a release fence would instead write back the whole L2.
+__device__ __forceinline__ void store1_rt_agent(void* base, int dtype, size_t idx, float v) {
+    switch (dtype) {
+        case DFLASH_F32: __hip_atomic_store(reinterpret_cast<float*>(base) + idx, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); break;
+        case DFLASH_BF16:
+            __hip_atomic_store(reinterpret_cast<uint16_t*>(base) + idx, f32_to_bf16_bits(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+        default:
+            __hip_atomic_store(reinterpret_cast<uint16_t*>(base) + idx, __builtin_bit_cast(uint16_t, (_Float16)v), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+            break;
+    }
+}
+__device__ __forceinline__ float load_agent(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_agent(const bf16_t* p) {
+    return to_float(bf16_t{__hip_atomic_load(reinterpret_cast<const uint16_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)});
+}
+__device__ __forceinline__ float load_agent(const f16_t* p) {
+    return (float)__builtin_bit_cast(_Float16, __hip_atomic_load(reinterpret_cast<const uint16_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+
+__device__ __forceinline__ float requant_rt(int dtype, float v) {      // v after a round trip through the type
+    switch (dtype) {
+        case DFLASH_F32: return v;
+        case DFLASH_BF16: return requant<bf16_t>(v);
+        default: return requant<f16_t>(v);
+    }
+}
+
 // ===========================================================================
 // Tape replay
 // ===========================================================================
@@ -382,8 +415,19 @@ struct GdnPrep {
     void* conv_out;           // [B,K-1,C]
     float q_scale, k_scale, eps;
     int C;
+    // The layer's post-op inside the same launch (all null / 0 when it is not asked for): the workgroup of a head
+    // that finishes last -- counted in arrivals[b*Hv + hv], which is zero before the launch and zero again after
+    // it -- normalises and gates the head's y rows.
+    const void* fin_gate;     // [B,T,Hv,Dv]
+    const void* fin_weight;   // [Dv]
+    void* fin_out;            // [B,T,Hv,Dv]; until the last workgroup writes a row, its first Dv/16 floats hold
+                              // the row tiles' sums of squares
+    int32_t* arrivals;        // [B*Hv]
+    float fin_eps;
+    int fin_silu;
 };
-constexpr int kLayerTaps = 4;  // conv kernel size the one-launch layer kernel is built for
+constexpr int kLayerTaps = 4;
+constexpr int kLayerFinishMaxDv = 256;   // head dim up to which the post-op runs inside the layer kernel  // conv kernel size the one-launch layer kernel is built for
 
 constexpr int kGdnChunk = 16;  // steps staged in LDS at a time
 
@@ -620,7 +664,9 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
                      "s"(A.Hv), "s"(A.Dv), "s"(P.x), "s"(P.conv_in), "s"(P.weight), "s"(P.a), "s"(P.b), "s"(P.a_log),
                      "s"(P.dt_bias), "s"(P.q_out), "s"(P.k_out), "s"(P.v_out), "s"(P.g_out), "s"(P.beta_out), "s"(P.conv_out),
                      "s"(P.q_scale), "s"(P.k_scale), "s"(P.eps), "s"(P.C));
-    else
+    if constexpr (FUSED)
+        asm volatile("" ::"s"(P.fin_gate), "s"(P.fin_weight), "s"(P.fin_out), "s"(P.arrivals), "s"(P.fin_eps), "s"(P.fin_silu));
+    if constexpr (!FUSED)
         asm volatile("" ::"s"(A.q), "s"(A.k), "s"(A.v), "s"(A.g), "s"(A.beta), "s"(A.mask), "s"(A.state_in), "s"(A.state_out),
                      "s"(A.y), "s"(A.tape), "s"(A.in_dtype), "s"(A.mask_dtype), "s"(A.T), "s"(A.Hk), "s"(A.Hv), "s"(A.Dv));
     constexpr int E = DK / 64;             // channels per lane in the state-update product (16 lanes x E x 4 waves = DK)
@@ -853,6 +899,39 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         }
     };
 
+    // out = rmsNorm(y; weight, eps) * act(gate) for the 16 steps x Dv channels of this head: thread (t, j) takes
+    // channels j, j + 16, ...; all of its loads go out together.
+    auto finish_head = [&](auto elem_tag, int tc) {
+        using Elem = decltype(elem_tag);
+        constexpr int MAXI = kLayerFinishMaxDv / 16;
+        const int t = ts < tc ? ts : tc - 1, tiles = (int)gridDim.x;
+        const size_t row = (((size_t)b * A.T + t) * A.Hv + hv) * A.Dv;
+        const Elem* yr = reinterpret_cast<const Elem*>(A.y) + row;
+        const Elem* zr = reinterpret_cast<const Elem*>(P.fin_gate) + row;
+        const Elem* wr = reinterpret_cast<const Elem*>(P.fin_weight);
+        Elem* orow = reinterpret_cast<Elem*>(P.fin_out) + row;
+        const float* part = reinterpret_cast<const float*>(orow);
+        float yv[MAXI], zv[MAXI], wv[MAXI], pp[MAXI];
+#pragma unroll
+        for (int i = 0; i < MAXI; ++i) {
+            const int d = tt + 16 * i, dl = d < A.Dv ? d : tt;
+            yv[i] = load_agent(yr + dl);
+            zv[i] = to_float(zr[dl]);
+            wv[i] = to_float(wr[dl]);
+            pp[i] = load_agent(part + (i < tiles ? i : 0));
+        }
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < MAXI; ++i)
+            if (i < tiles) ss = __fadd_rn(ss, pp[i]);
+        const float inv = gdn_rms_inv(ss, A.Dv, P.fin_eps);
+#pragma unroll
+        for (int i = 0; i < MAXI; ++i) {
+            const int d = tt + 16 * i;
+            if (d < A.Dv && ts < tc) orow[d] = from_float<Elem>(gdn_gated_out(yv[i], inv, wv[i], zv[i], P.fin_silu != 0));
+        }
+    };
+
     // One chunk of up to 16 steps.  The first chunk (the only one of a verify block) is straight-line code ahead of
     // the loop over the rest: inside the loop the compiler hoists every invariant of the whole body above the first
     // load and carries waits round the back edge.
@@ -946,10 +1025,24 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
             float yv = L.gam[t] * L.p[r][16 + t];
 #pragma unroll
             for (int s = 0; s < kChunkSteps; ++s) yv = fmaf(L.c[s][t], L.dl[s][r], yv);
+            yv = L.on[t] ? yv : 0.f;
             if (t < tc) {
                 const size_t o = (((size_t)b * A.T + t0 + t) * A.Hv + hv) * A.Dv + row0 + r;
-                store1_rt(A.y, A.in_dtype, o, L.on[t] ? yv : 0.f);
+                if (FUSED && P.fin_gate) store1_rt_agent(A.y, A.in_dtype, o, yv);   // re-read by the head's last workgroup
+                else store1_rt(A.y, A.in_dtype, o, yv);
                 A.tape[o] = L.dl[t][r];
+            }
+            if constexpr (FUSED) {
+                if (P.fin_gate) {          // this tile's share of sum(y^2) of step t, parked in the row of `out`
+                    const float yq = requant_rt(A.in_dtype, yv);
+                    const float sq = group_sum<16>(__fmul_rn(yq, yq));
+                    if (r == 0 && t < tc) {
+                        const size_t row = ((size_t)b * A.T + t) * A.Hv + hv;
+                        const size_t esz = A.in_dtype == DFLASH_F32 ? 4 : 2;
+                        __hip_atomic_store(reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(P.fin_out) + row * A.Dv * esz) + blockIdx.x,
+                                           sq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                }
             }
         }
 
@@ -990,6 +1083,25 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
                     asm volatile("" ::: "memory");
                 }
                 // the staging barrier of the next chunk orders these writes before their readers
+            }
+        }
+
+        // ---- the layer's post-op, by the head's last workgroup ----
+        // Every workgroup of the head has written its y rows and sums of squares through to agent scope; once those
+        // stores are acknowledged it counts itself in, and the one that finds all others already counted re-reads
+        // the head's y (at agent scope), finishes the sums and writes `out`.  Nothing waits for anything: a
+        // workgroup that is not last is done.
+        if constexpr (FUSED) {
+            if (P.fin_gate) {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                if (tid == 0) L.on[0] = __hip_atomic_fetch_add(P.arrivals + bh, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __syncthreads();
+                if (L.on[0] != (int)gridDim.x - 1) return;
+                if (tid == 0) __hip_atomic_store(P.arrivals + bh, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // as the next launch expects it
+                if (A.in_dtype == DFLASH_BF16) finish_head(bf16_t{}, tc);
+                else if (A.in_dtype == DFLASH_F16) finish_head(f16_t{}, tc);
+                else finish_head(float{}, tc);
             }
         }
     };
@@ -1157,8 +1269,8 @@ extern "C" int dflash_gdn_layer(void* stream, const void* mixed_qkv, const void*
                                 int in_dtype, float q_scale, float k_scale, float norm_eps, const void* state_in,
                                 void* state_out, void* k_out, void* g_out, float* tape_out, void* conv_state_out,
                                 void* y_out, const void* gate, const void* out_norm_weight, float out_norm_eps,
-                                int gate_kind, void* out, void* q_out, void* v_out, void* beta_out, int B, int T, int Hk,
-                                int Hv, int Dk, int Dv, int K) {
+                                int gate_kind, void* out, int32_t* arrivals, void* q_out, void* v_out, void* beta_out,
+                                int B, int T, int Hk, int Hv, int Dk, int Dv, int K) {
     int rc = ensure_init();
     if (rc) return rc;
     DFLASH_REQUIRE(B > 0 && T > 0 && Hk > 0 && Hv > 0 && Dk > 0 && Dv > 0, "gdn_layer: non-positive dimension");
@@ -1168,6 +1280,7 @@ extern "C" int dflash_gdn_layer(void* stream, const void* mixed_qkv, const void*
     DFLASH_REQUIRE(state_in != state_out, "gdn_layer: state_in aliases state_out");
     DFLASH_REQUIRE(conv_state_out != conv_state_in, "gdn_layer: conv_state_out aliases conv_state_in");
     DFLASH_REQUIRE(!gate || (out_norm_weight && out), "gdn_layer: a gate needs out_norm_weight and out");
+    DFLASH_REQUIRE(!gate || out != y_out, "gdn_layer: out aliases y_out");
     DFLASH_REQUIRE(gate_kind == 0 || gate_kind == 1, "gdn_layer: gate_kind must be 0 (sigmoid) or 1 (silu)");
     DFLASH_REQUIRE((long)B * Hv <= 65535, "gdn_layer: B*Hv too large for one launch");
     DFLASH_SUPPORTED(in_dtype == DFLASH_F32 || in_dtype == DFLASH_BF16 || in_dtype == DFLASH_F16, "gdn_layer: bad in_dtype %d", in_dtype);
@@ -1184,10 +1297,19 @@ extern "C" int dflash_gdn_layer(void* stream, const void* mixed_qkv, const void*
     P.a_log = a_log; P.dt_bias = dt_bias; P.q_out = q_out; P.k_out = k_out; P.v_out = v_out; P.g_out = g_out;
     P.beta_out = beta_out; P.conv_out = conv_state_out; P.q_scale = q_scale; P.k_scale = k_scale; P.eps = norm_eps;
     P.C = 2 * Hk * Dk + Hv * Dv;
+    // With a counter array the post-op runs inside the same launch; without one (or with a head dim the kernel's
+    // post-op is not unrolled for) it is a second launch.
+    const bool finish_inside = gate && arrivals && Dv <= kLayerFinishMaxDv;
+    P.fin_gate = finish_inside ? gate : nullptr;
+    P.fin_weight = finish_inside ? out_norm_weight : nullptr;
+    P.fin_out = finish_inside ? out : nullptr;
+    P.arrivals = finish_inside ? arrivals : nullptr;
+    P.fin_eps = out_norm_eps;
+    P.fin_silu = gate_kind;
     hipStream_t st = (hipStream_t)stream;
     if (Dk == 64) rc = launch_gdn_layer<64>(st, A, P, B);
     else if (Dk == 128) rc = launch_gdn_layer<128>(st, A, P, B);
     else rc = launch_gdn_layer<256>(st, A, P, B);
-    if (rc || !gate) return rc;
+    if (rc || !gate || finish_inside) return rc;
     return dflash_gdn_finish(stream, y_out, gate, out_norm_weight, out, in_dtype, out_norm_eps, gate_kind, B, T, Hv, Dv);
 }

@@ -149,24 +149,30 @@ __global__ __launch_bounds__(256) void gdn_finish_kernel(FinishArgs A) {
     const Elem* wt = reinterpret_cast<const Elem*>(A.weight);
     Elem* out = reinterpret_cast<Elem*>(A.out) + (size_t)row * A.Dv;
     constexpr int kMaxPer = 16;                      // Dv <= 1024
-    float v[kMaxPer];
-    float ss = 0.f;
+    float v[kMaxPer], part[kMaxPer];
 #pragma unroll
     for (int i = 0; i < kMaxPer; ++i) {
         const int d = lane + 64 * i;
         v[i] = d < A.Dv ? to_float(y[d]) : 0.f;
-        ss = fmaf(v[i], v[i], ss);
+        part[i] = group_sum<16>(__fmul_rn(v[i], v[i]));      // channels 64 i + 16 (lane / 16) .. + 15
     }
-    for (int o = 32; o >= 1; o >>= 1) ss += __shfl_xor(ss, o);
-    const float inv = rsqrtf(ss / (float)A.Dv + A.eps);
+    // the 16-channel sums in channel order (group g of pass i holds channels 64 i + 16 g ..)
+    const int tiles = (A.Dv + 15) / 16;
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxPer; ++i) {
+        if (4 * i >= tiles) break;                   // uniform
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const float p = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(part[i]), 16 * g));
+            if (4 * i + g < tiles) ss = __fadd_rn(ss, p);
+        }
+    }
+    const float inv = gdn_rms_inv(ss, A.Dv, A.eps);
 #pragma unroll
     for (int i = 0; i < kMaxPer; ++i) {
         const int d = lane + 64 * i;
-        if (d < A.Dv) {
-            const float z = to_float(gt[d]);
-            const float act = A.silu_gate ? z * sigmoid_f(z) : sigmoid_f(z);
-            out[d] = from_float<Elem>(v[i] * inv * to_float(wt[d]) * act);
-        }
+        if (d < A.Dv) out[d] = from_float<Elem>(gdn_gated_out(v[i], inv, to_float(wt[d]), to_float(gt[d]), A.silu_gate != 0));
     }
 }
 

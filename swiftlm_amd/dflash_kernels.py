@@ -22,6 +22,10 @@ _DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F
        torch.uint8: _lib.U8, torch.bool: _lib.U8}
 
 
+# arrival counters of gdn_layer's in-launch gated norm: int32 zeros per (device, stream, B*Hv), left zero by every call
+_ARRIVALS = {}
+
+
 def _code(t: torch.Tensor) -> int:
     try:
         return _DT[t.dtype]
@@ -193,13 +197,19 @@ class DFlashKernels:
                   a_logits: torch.Tensor, b_logits: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
                   state: torch.Tensor, Hk: int, Hv: int, Dk: int, Dv: int, q_scale: float, k_scale: float,
                   eps: float = 1e-6, gate: Optional[torch.Tensor] = None, norm_weight: Optional[torch.Tensor] = None,
-                  norm_eps: float = 1e-6, gate_kind: str = "sigmoid", want_intermediates: bool = False):
+                  norm_eps: float = 1e-6, gate_kind: str = "sigmoid", want_intermediates: bool = False,
+                  arrivals: Optional[torch.Tensor] = None, one_launch: bool = True):
         """The body of a GatedDelta layer between its projections (KimiLinearDFlash.swift:351-378) in one
         call: ``gdn_prepare`` -> ``gated_delta_kernel_with_tape`` -> ``gdn_finish`` with the pre-ops done
         inside the forward kernel.  Returns a dict: ``out`` (None without ``gate``), ``y``, ``state``,
         ``tape``, ``k``, ``g`` (what ``record_tape`` keeps), ``conv_state``, and with
         ``want_intermediates`` also ``q``, ``v``, ``beta``.  Raises DFlashUnsupported outside the verify
-        block's case (float32 state, scalar gate, K == 4, T <= 16), where the three calls apply."""
+        block's case (float32 state, scalar gate, K == 4, T <= 16), where the three calls apply.
+
+        With a ``gate`` the gated norm runs inside the same launch, done by the last workgroup of each head;
+        the heads' arrival counters are ``arrivals`` (int32 [B*Hv], zero before and after every call) or, when
+        it is None, an array this module keeps per device, stream and size.  ``one_launch=False`` runs the gated
+        norm as a second launch instead."""
         _dev(mixed_qkv, conv_state, conv_weight, a_logits, b_logits, a_log, dt_bias, state, gate, norm_weight)
         B, T, C = mixed_qkv.shape
         if C != 2 * Hk * Dk + Hv * Dv:
@@ -234,11 +244,22 @@ class DFlashKernels:
                 raise DFlashError("gdn_layer: gate must be [B,T,Hv,Dv] and come with norm_weight [Dv]")
             zg, nw = gate.to(dt).contiguous(), norm_weight.to(dt).contiguous()
             out = torch.empty_like(y)
+            if not one_launch:
+                arrivals = None
+            elif arrivals is None:
+                key = (dv.index, torch.cuda.current_stream().cuda_stream, B * Hv)
+                arrivals = _ARRIVALS.get(key)
+                if arrivals is None:
+                    arrivals = _ARRIVALS[key] = torch.zeros(B * Hv, dtype=torch.int32, device=dv)
+            elif arrivals.dtype != torch.int32 or arrivals.numel() < B * Hv or not arrivals.is_contiguous():
+                raise DFlashError("gdn_layer: arrivals must be a contiguous int32 tensor of at least B*Hv elements")
+        else:
+            arrivals = None
         rc = _lib.load().dflash_gdn_layer(
             _stream(), _ptr(x), _ptr(st), _ptr(w), _ptr(a), _ptr(bl), _ptr(al), _ptr(db), _code(x),
             float(q_scale), float(k_scale), float(eps), _ptr(state), _ptr(new_state), _ptr(k), _ptr(g), _ptr(tape),
             _ptr(new_conv), _ptr(y), _ptr(zg), _ptr(nw), float(norm_eps), {"sigmoid": 0, "silu": 1}[gate_kind],
-            _ptr(out), _ptr(q), _ptr(v), _ptr(beta), B, T, Hk, Hv, Dk, Dv, K)
+            _ptr(out), _ptr(arrivals), _ptr(q), _ptr(v), _ptr(beta), B, T, Hk, Hv, Dk, Dv, K)
         _lib.check(rc, "gdn_layer")
         res = dict(out=out, y=y, state=new_state, tape=tape, k=k, g=g, conv_state=new_conv)
         if want_intermediates:

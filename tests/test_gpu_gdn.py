@@ -360,12 +360,20 @@ def test_gdn_layer_equals_prepare_forward_finish_bitwise(gpu_lib, cfg, in_dt, ca
     q, k, v, g, beta, conv1 = K.gdn_prepare(x, st, w, a, bl, dev(d["a_log"]), dev(d["dt_bias"]), Hk, Hv, Dk, Dv, **sc)
     y, s1, tape = K.gated_delta_kernel_with_tape(q, k, v, g, beta, s0)
     out = K.gdn_finish(y, z, nw, 1e-6, "silu")
-    r = K.gdn_layer(x, st, w, a, bl, dev(d["a_log"]), dev(d["dt_bias"]), s0, Hk, Hv, Dk, Dv, **sc, gate=z, norm_weight=nw,
-                    norm_eps=1e-6, gate_kind="silu", want_intermediates=True)
+    # the gated norm inside the launch (twice with one counter array: the call must leave it zeroed), and as a
+    # second launch
+    arrivals = torch.zeros(B * Hv, dtype=torch.int32, device="cuda")
+    layer_args = (x, st, w, a, bl, dev(d["a_log"]), dev(d["dt_bias"]), s0, Hk, Hv, Dk, Dv)
+    layer_kw = dict(**sc, gate=z, norm_weight=nw, norm_eps=1e-6, gate_kind="silu", want_intermediates=True)
+    runs = [K.gdn_layer(*layer_args, **layer_kw, arrivals=arrivals), K.gdn_layer(*layer_args, **layer_kw, arrivals=arrivals),
+            K.gdn_layer(*layer_args, **layer_kw, one_launch=False)]
     torch.cuda.synchronize()
-    for name, want in (("q", q), ("k", k), ("v", v), ("g", g), ("beta", beta), ("conv_state", conv1), ("y", y),
-                       ("state", s1), ("tape", tape), ("out", out)):
-        assert torch.equal(r[name], want), name
+    assert not arrivals.any()
+    for r in runs:
+        for name, want in (("q", q), ("k", k), ("v", v), ("g", g), ("beta", beta), ("conv_state", conv1), ("y", y),
+                           ("state", s1), ("tape", tape), ("out", out)):
+            assert torch.equal(r[name], want), name
+    r = runs[0]
     # without the optional outputs and without a gate: same recurrence results
     r2 = K.gdn_layer(x, st, w, a, bl, dev(d["a_log"]), dev(d["dt_bias"]), s0, Hk, Hv, Dk, Dv, **sc)
     torch.cuda.synchronize()
