@@ -239,41 +239,41 @@ class StepChecker:
         return errs
 
 
-def launch_floor(lib, stack, reps=50):
+def launch_floor(lib, stack, steps_per_graph, replays):
     """What the launches of a step cost before any work: a HIP graph of empty kernels with the grid, block and
-    LDS size of every kernel of two steps (the timed graphs hold two steps as well), replayed `reps` times
-    between host-clock reads.  Returns microseconds per step and the launch count per step."""
+    LDS size of every kernel of `steps_per_graph` steps (as many as a timed graph holds), replayed `replays`
+    times between host-clock reads.  Returns microseconds per step and the launch count per step."""
     import torch
 
     shapes = stack.launch_shapes()
     side = torch.cuda.Stream()
+
+    def _check(rc):
+        if rc != 0:
+            raise RuntimeError("dflash_profile_empty_launch: status %d: %s" % (rc, lib.dflash_last_error().decode()))
 
     def enqueue():
         st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
         for gx, gy, gz, threads, lds in shapes:
             _check(lib.dflash_profile_empty_launch(st, gx, gy, gz, threads, lds))
 
-    def _check(rc):
-        if rc != 0:
-            raise RuntimeError("dflash_profile_empty_launch: status %d: %s" % (rc, lib.dflash_last_error().decode()))
-
     enqueue()
     torch.cuda.synchronize()
     side.wait_stream(torch.cuda.current_stream())
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g, stream=side):
-        enqueue()
-        enqueue()
+        for _ in range(steps_per_graph):
+            enqueue()
     torch.cuda.current_stream().wait_stream(side)
-    for _ in range(5):
+    for _ in range(3):
         g.replay()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(reps):
+    for _ in range(replays):
         g.replay()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    return dt / (2 * reps) * 1e6, len(shapes)
+    return dt / (steps_per_graph * replays) * 1e6, len(shapes)
 
 
 def aux_kernels(lib, cfg, reps=48):
@@ -688,7 +688,9 @@ def main():
         print(json.dumps({"metric": "dflash_verify_us_per_layer", "verified": False, "error": str(e)[:400]}))
         sys.exit(1)
 
-    floor_us, n_launches = launch_floor(lib, stack)
+    floor_graph = 2 if args.no_graph else G
+    floor_replays = max(4, 100 // floor_graph)
+    floor_us, n_launches = launch_floor(lib, stack, floor_graph, floor_replays)
 
     mean_commit = int(round(float(np.mean(commits))))
     step_bytes = n_gdn * (stack.gdn_forward_bytes() + stack.replay_bytes(mean_commit)) + n_attn * sdpa_bytes
@@ -723,7 +725,8 @@ def main():
         "step_frac_of_hbm_peak": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "launch_floor": {
             "us_per_step": round(floor_us, 1), "launches_per_step": n_launches, "us_per_launch": round(floor_us / n_launches, 2),
-            "how": "HIP graph of empty kernels with every step kernel's grid, block and LDS size, in one chain, two steps per graph, 50 replays",
+            "how": "HIP graph of empty kernels with every step kernel's grid, block and LDS size, in one chain, %d steps per graph, %d replays"
+                   % (floor_graph, floor_replays),
         },
         "step_minus_floor_ms": round(ms_per_step - floor_us * 1e-3, 4),
         "step_frac_of_hbm_peak_above_floor": round(step_bytes / ((ms_per_step - floor_us * 1e-3) * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
