@@ -617,8 +617,7 @@ template <int DK> struct GdnChunkLds {
     static constexpr int LD = DK + 4;      // row pitch in floats: 16-byte pad spreads rows over the banks
     float x[32][LD];                       // rows 0..15 state tile, rows 16..31 k_t
     float y[32][LD];                       // rows 0..15 k_t, rows 16..31 q_t
-    float red[4][32][33];                  // per-wave partial products (each wave contracts Dk/4 channels)
-    float p[32][33];                       // [S_0 ; k] x [k | q]^T
+    float p[16][33];                       // S_0 x [k | q]^T: p[r][t] = S_0 k_t, p[r][16 + t] = S_0 q_t of state row r
     float a[16][16];                       // a[s][t] = G[s][t] k_s.k_t for s < t, else 0
     float c[16][16];                       // c[s][t] = G[s][t] k_s.q_t for s <= t, else 0
     float dl[16][17];                      // delta_s of row r at dl[s][r]
@@ -949,53 +948,91 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         }
         __syncthreads();
 
-        // ---- [S_0 ; k] x [k | q]^T, wave w contracting channels w*DK/4 .. +DK/4-1 ----
-        // A 32x32x2 fp32 MFMA takes lane l's a as row l%32, contraction index l/32 (b alike), so a float4
-        // per lane feeds four MFMAs whose index pairs are {e, 4+e} of an 8-channel group.
-        float G = 1.f;                      // decay product of the pair (s, t) = (ts, tt)
+        // ---- [S_0 ; k] x [k | q]^T: one 16x16 block per wave, over all DK channels ----
+        //   wave 0: S_0 k_t -> p[r][t]     wave 1: S_0 q_t -> p[r][16+t]     wave 2: k_s.k_t -> a     wave 3: k_s.q_t -> c
+        // A 16x16x4 fp32 MFMA takes lane l's a as row l%16, contraction index l/16 (b alike) and leaves lane l with
+        // column l%16, rows 4*(l/16)+v; a float4 per lane feeds four MFMAs whose index sets are {16c + 4*(l/16) + e}.
+        // No reduction across waves: the block's coefficients go from the accumulators straight into the tables.
         {
-            f32x16v acc;
+            const int n = lane % 16, kk = lane / 16;
+            const int ws = __builtin_amdgcn_readfirstlane(w);
+            const float* ap = &L.x[(ws < 2 ? 0 : 16) + n][4 * kk];
+            const float* bp = &L.y[(ws & 1 ? 16 : 0) + n][4 * kk];
+            constexpr int NB = DK / 16, PS = 4 * NB / 16;     // 4*NB MFMAs, 15 pieces
+            float4 av[NB], bv[NB];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-            const int kc0 = w * (DK / 4) + 4 * (lane / 32);
-#pragma unroll
-            for (int c = 0; c < DK / 32; ++c) {
-                const float4 a4 = *reinterpret_cast<const float4*>(&L.x[lane % 32][kc0 + 8 * c]);
-                const float4 b4 = *reinterpret_cast<const float4*>(&L.y[lane % 32][kc0 + 8 * c]);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.x, b4.x, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.y, b4.y, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.z, b4.z, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.w, b4.w, acc, 0, 0, 0);
+            for (int c = 0; c < NB; ++c) {
+                av[c] = *reinterpret_cast<const float4*>(ap + 16 * c);
+                bv[c] = *reinterpret_cast<const float4*>(bp + 16 * c);
             }
-            // The decay products run in the shadow of the MFMAs (the matrix pipe is busy for a thousand cycles after
-            // the last one is issued): all 16 decays are read unconditionally, four at a time, and selected in
-            // registers -- a conditional read per step costs an exec-mask round trip each.
-            __builtin_amdgcn_sched_barrier(0);
-            {
-                float gj[kChunkSteps];
+            float gj[kChunkSteps];
 #pragma unroll
-                for (int j4 = 0; j4 < kChunkSteps; j4 += 4) {
-                    const float4 g4 = *reinterpret_cast<const float4*>(&L.g[j4]);
-                    gj[j4] = g4.x; gj[j4 + 1] = g4.y; gj[j4 + 2] = g4.z; gj[j4 + 3] = g4.w;
+            for (int j4 = 0; j4 < kChunkSteps; j4 += 4) {
+                const float4 g4 = *reinterpret_cast<const float4*>(&L.g[j4]);
+                gj[j4] = g4.x; gj[j4 + 1] = g4.y; gj[j4 + 2] = g4.z; gj[j4 + 3] = g4.w;
+            }
+            // The decay products G[v] = g_{s+1} ... g_t of the lane's pairs (s, t) = (4*kk + v, n) (1 where s >= t)
+            // are computed one factor at a time between the MFMAs: an instruction issued right behind an MFMA runs
+            // while the matrix pipe works, one issued behind the last MFMA is on the critical path.  Piece i:
+            // 0..11 the factors j = 4..15 of G[3], 12..14 one more factor for G[2], G[1], G[0], 15 the table
+            // coefficients (a[s][t] = G k_s.k_t for s < t, c[s][t] = G k_s.q_t for s <= t, else 0).  All 16 decays
+            // are read unconditionally and selected in registers.
+            float G[4] = {1.f, 1.f, 1.f, 1.f}, coef[4];
+            const int pitch = ws < 2 ? 33 : 16;
+            float* const lds_f = reinterpret_cast<float*>(gdn_chunk_smem);
+            int tbl = (int)((ws == 0 ? &L.p[0][0] : ws == 1 ? &L.p[0][16] : ws == 2 ? &L.a[0][0] : &L.c[0][0]) - &L.x[0][0]) +
+                      4 * kk * pitch + n;               // float index of the lane's first table entry in LDS
+            asm volatile("" : "+v"(tbl));
+            auto g_piece = [&](int i) {
+                if (i < 12) {
+                    const int j = i + 4;
+                    G[3] *= (j > 4 * kk + 3 && j <= n) ? gj[j] : 1.f;
+                    asm volatile("" : "+v"(G[3]));   // pins the piece where it is written (the optimiser would sink it)
+                } else if (i < 15) {
+                    const int v = 14 - i;           // 2, 1, 0: g_{s+1} with s = 4*kk + v
+                    float gs = 1.f;
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4) gs = kk == q4 ? gj[4 * q4 + v + 1] : gs;
+                    G[v] = G[v + 1] * (4 * kk + v + 1 <= n ? gs : 1.f);
+                    asm volatile("" : "+v"(G[v]));
+                } else if (i == 15) {               // what the block's entries are multiplied by on their way to the tables
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int s = 4 * kk + v;
+                        const bool keep = ws == 2 ? s < n : s <= n;
+                        coef[v] = ws < 2 ? 1.f : (keep ? G[v] : 0.f);
+                        asm volatile("" : "+v"(coef[v]));
+                    }
                 }
-#pragma unroll
-                for (int j = 1; j < kChunkSteps; ++j) G *= (j > ts && j <= tt) ? gj[j] : 1.f;
-            }
+            };
+            f32x4v acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int v = 0; v < 16; ++v) L.red[w][8 * (v / 4) + 4 * (lane / 32) + (v % 4)][lane % 32] = acc[v];
-        }
-        __syncthreads();
-        // sum the four partial products: the S_0 half (16 x 32) as two entries per thread, the k half
-        // straight into the coefficient tables of the pair (ts, tt)
-        {
-            auto red4 = [&](int r, int c) { return (L.red[0][r][c] + L.red[1][r][c]) + (L.red[2][r][c] + L.red[3][r][c]); };
-            L.p[ts][tt] = red4(ts, tt);
-            L.p[ts][16 + tt] = red4(ts, 16 + tt);
-            L.a[ts][tt] = ts < tt ? G * red4(16 + ts, tt) : 0.f;
-            L.c[ts][tt] = ts <= tt ? G * red4(16 + ts, 16 + tt) : 0.f;
-            if (ts == 0) L.gam[tt] = L.g[0] * G;
-            if (tt == kChunkSteps - 1) L.w[ts] = G;
+            for (int c = 0; c < NB; c += 2) {
+                const float a0[4] = {av[c].x, av[c].y, av[c].z, av[c].w}, b0[4] = {bv[c].x, bv[c].y, bv[c].z, bv[c].w};
+                const float a1[4] = {av[c + 1].x, av[c + 1].y, av[c + 1].z, av[c + 1].w};
+                const float b1[4] = {bv[c + 1].x, bv[c + 1].y, bv[c + 1].z, bv[c + 1].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int m = 4 * c + 2 * e;            // MFMA number; a piece behind every PS-th
+                    acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[e], b0[e], acc0, 0, 0, 0);
+                    g_piece(m % PS == 0 ? m / PS : 100);
+                    __builtin_amdgcn_sched_barrier(0);
+                    acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[e], b1[e], acc1, 0, 0, 0);
+                    g_piece((m + 1) % PS == 0 ? (m + 1) / PS : 100);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            // row 4*kk + v of the block: a state row (waves 0, 1) or step s (waves 2, 3); column n
+#pragma unroll
+            for (int v = 0; v < 4; ++v) lds_f[tbl + v * pitch] = coef[v] * (acc0[v] + acc1[v]);
+            if (ws == 3) {
+                if (kk == 0) L.gam[n] = gj[0] * G[0];
+                if (n == kChunkSteps - 1) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) L.w[4 * kk + v] = G[v];
+                }
+            }
         }
         __syncthreads();
 
