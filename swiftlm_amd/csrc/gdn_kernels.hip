@@ -399,6 +399,9 @@ struct GdnArgs {
     float* tape;
     int in_dtype, mask_dtype;
     int T, Hk, Hv, Dv;
+    // chunked kernels only: value heads per key head and ceil(2^32 / group), so that hv / group is one multiply
+    // (exact for hv, group < 2^16; group == 1 is handled apart, its reciprocal does not fit)
+    uint32_t group, group_magic;
 };
 
 // Inputs of the layer's pre-ops when they run inside the forward kernel (gdn_layer_kernel): the short
@@ -660,24 +663,29 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
     // cache line of the argument block is a trip to memory on the way to the first global load.
     if constexpr (FUSED)
         asm volatile("" ::"s"(A.state_in), "s"(A.state_out), "s"(A.y), "s"(A.tape), "s"(A.in_dtype), "s"(A.T), "s"(A.Hk),
-                     "s"(A.Hv), "s"(A.Dv), "s"(P.x), "s"(P.conv_in), "s"(P.weight), "s"(P.a), "s"(P.b), "s"(P.a_log),
+                     "s"(A.Hv), "s"(A.Dv), "s"(A.group), "s"(A.group_magic), "s"(P.x), "s"(P.conv_in), "s"(P.weight), "s"(P.a), "s"(P.b), "s"(P.a_log),
                      "s"(P.dt_bias), "s"(P.q_out), "s"(P.k_out), "s"(P.v_out), "s"(P.g_out), "s"(P.beta_out), "s"(P.conv_out),
                      "s"(P.q_scale), "s"(P.k_scale), "s"(P.eps), "s"(P.C));
     if constexpr (FUSED)
         asm volatile("" ::"s"(P.fin_gate), "s"(P.fin_weight), "s"(P.fin_out), "s"(P.arrivals), "s"(P.fin_eps), "s"(P.fin_silu));
     if constexpr (!FUSED)
         asm volatile("" ::"s"(A.q), "s"(A.k), "s"(A.v), "s"(A.g), "s"(A.beta), "s"(A.mask), "s"(A.state_in), "s"(A.state_out),
-                     "s"(A.y), "s"(A.tape), "s"(A.in_dtype), "s"(A.mask_dtype), "s"(A.T), "s"(A.Hk), "s"(A.Hv), "s"(A.Dv));
+                     "s"(A.y), "s"(A.tape), "s"(A.in_dtype), "s"(A.mask_dtype), "s"(A.T), "s"(A.Hk), "s"(A.Hv), "s"(A.Dv),
+                     "s"(A.group), "s"(A.group_magic));
     constexpr int E = DK / 64;             // channels per lane in the state-update product (16 lanes x E x 4 waves = DK)
     static_assert(DK % 64 == 0, "chunked gated delta needs Dk to be a multiple of 64");
 
     const int tid = threadIdx.x, lane = tid % 64, w = tid / 64;
-    const int bh = blockIdx.y;
-    const int b = bh / A.Hv, hv = bh % A.Hv;
-    const int hk = hv / (A.Hv / A.Hk);
+    // Grid (Dv/16, Hv, B): no division on the way to the first address (an integer division is some twenty
+    // dependent instructions, and everything ahead of the loads is on the critical path).  Element offsets into
+    // q/k/v/g/beta/y/tape are 32-bit (the host checks the sizes), their per-thread parts 24-bit multiplies.
+    const int b = blockIdx.z, hv = blockIdx.y;
+    const int bh = b * A.Hv + hv;
+    const int hk = A.group == 1 ? hv : (int)__umulhi((uint32_t)hv, A.group_magic);
     const int row0 = blockIdx.x * kChunkRows;
     const float* s_in = reinterpret_cast<const float*>(A.state_in) + ((size_t)bh * A.Dv + row0) * DK;
     float* s_out = reinterpret_cast<float*>(A.state_out) + ((size_t)bh * A.Dv + row0) * DK;
+    const uint32_t k_step = (uint32_t)A.Hk * DK, v_step = (uint32_t)A.Hv * A.Dv;       // elements per step
 
     constexpr int NV = kChunkRows * (DK / 4) / kThreads;      // float4 groups per thread of a 16 x DK tile
     const int ts = tid / 16, tt = tid % 16;        // (s, t) for the tables, (t, r) for v / y / tape
@@ -697,7 +705,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
         const int i = tid + u * kThreads, r = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
-        sv0[u] = load4(s_in + (size_t)r * DK + c4);
+        sv0[u] = load4(s_in + (uint32_t)(r * DK + c4));
     }
 
     // Stage one chunk: every global load of the chunk (the state tile is already on its way) is issued
@@ -712,24 +720,26 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         const Elem* bp = reinterpret_cast<const Elem*>(A.beta);
         float4 kv[NV], qv[NV];
         const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        const uint32_t bt0 = (uint32_t)b * A.T + t0;                       // first step of the chunk, all uniform
+        const uint32_t k0 = (bt0 * A.Hk + hk) * DK, v0 = (bt0 * A.Hv + hv) * A.Dv + row0, g0 = bt0 * A.Hv + hv;
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
             const int i = tid + u * kThreads, t = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
             const int tl = t < tc ? t : tc - 1;           // clamped: always a valid address, selected away below
-            const size_t o = (((size_t)b * A.T + t0 + tl) * A.Hk + hk) * DK + c4;
+            const uint32_t o = k0 + __umul24(tl, k_step) + c4;
             kv[u] = load4(kp + o);
             qv[u] = load4(qp + o);
         }
         const int tvl = ts < tc ? ts : tc - 1;
-        const float vv = to_float(vp[(((size_t)b * A.T + t0 + tvl) * A.Hv + hv) * A.Dv + row0 + tt]);
+        const float vv = to_float(vp[v0 + __umul24(tvl, v_step) + tt]);
         float gv = 1.f, bv = 0.f;
         bool on = false;
         if (tid < kChunkSteps) {
             const int tl = tid < tc ? tid : tc - 1;
-            const size_t bt = (size_t)b * A.T + t0 + tl;
-            gv = to_float(gp[bt * A.Hv + hv]);
-            bv = to_float(bp[bt * A.Hv + hv]);
-            on = HAS_MASK ? mask_on(A.mask, A.mask_dtype, (int)bt) : true;
+            const uint32_t go = g0 + __umul24(tl, A.Hv);
+            gv = to_float(gp[go]);
+            bv = to_float(bp[go]);
+            on = HAS_MASK ? mask_on(A.mask, A.mask_dtype, (int)(bt0 + tl)) : true;
             on = on && tid < tc;
         }
         if (with_state) {
@@ -778,14 +788,14 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         auto win_row = [&](int r) -> const Elem* {
             const bool in_x = r >= keep;
             const int rr = in_x ? r - keep : (cs ? r : 0);
-            return (in_x ? x : csz) + (size_t)rr * C;
+            return (in_x ? x : csz) + __umul24(rr, C);
         };
         float4 kw[NV][KT], qw[NV][KT], ktap[4], qtap[4], vtap;
         float vw[KT];
 #pragma unroll
         for (int m = 0; m < 4; ++m) {               // [m] = the KT taps of channel c4 + m
-            ktap[m] = load4(wt + (size_t)(ck + c4 + m) * KT);
-            qtap[m] = load4(wt + (size_t)(cq + c4 + m) * KT);
+            ktap[m] = load4(wt + (uint32_t)((ck + c4 + m) * KT));
+            qtap[m] = load4(wt + (uint32_t)((cq + c4 + m) * KT));
         }
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
@@ -800,10 +810,10 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         const int tvl = ts < tc ? ts : tc - 1;
 #pragma unroll
         for (int j = 0; j < KT; ++j) vw[j] = to_float(win_row(tvl + j)[cv + tt]);
-        vtap = load4(wt + (size_t)(cv + tt) * KT);
+        vtap = load4(wt + (uint32_t)((cv + tt) * KT));
         // gate inputs: every thread reads them (step tid mod 16), so that no load sits inside a branch
         const int tg = (tid % kChunkSteps) < tc ? (tid % kChunkSteps) : tc - 1;
-        const size_t btg = ((size_t)b * A.T + tg) * A.Hv + hv;
+        const uint32_t btg = ((uint32_t)b * A.T + tg) * A.Hv + hv;
         const float av = to_float(reinterpret_cast<const Elem*>(P.a)[btg]);
         const float bv = to_float(reinterpret_cast<const Elem*>(P.b)[btg]);
         const float alog = P.a_log[hv];
@@ -1064,7 +1074,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
             for (int s = 0; s < kChunkSteps; ++s) yv = fmaf(L.c[s][t], L.dl[s][r], yv);
             yv = L.on[t] ? yv : 0.f;
             if (t < tc) {
-                const size_t o = (((size_t)b * A.T + t0 + t) * A.Hv + hv) * A.Dv + row0 + r;
+                const uint32_t o = (((uint32_t)b * A.T + t0) * A.Hv + hv) * A.Dv + row0 + __umul24(t, v_step) + r;
                 if (FUSED && P.fin_gate) store1_rt_agent(A.y, A.in_dtype, o, yv);   // re-read by the head's last workgroup
                 else store1_rt(A.y, A.in_dtype, o, yv);
                 A.tape[o] = L.dl[t][r];
@@ -1107,7 +1117,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
 #pragma unroll
-                    for (int e = 0; e < E; ++e) s_out[(size_t)(4 * kk + v) * DK + base + e] = cacc[e][v];
+                    for (int e = 0; e < E; ++e) s_out[(uint32_t)((4 * kk + v) * DK + base + e)] = cacc[e][v];
             } else {
                 __syncthreads();           // every wave has read the old tile
                 // One row at a time, with a compiler barrier between the rows: when the stores of rows 2 and 3 are
@@ -1158,10 +1168,21 @@ __global__ __launch_bounds__(kThreads) void gdn_layer_kernel(GdnArgs A, GdnPrep 
     gdn_chunk_body<false, DK, true>(A, P);
 }
 
+// Whether the chunked kernels' 32-bit element offsets and 24-bit per-step strides cover this shape, and the
+// reciprocal of the head group for them.
+static bool chunk_index_setup(GdnArgs& A, int B, int Dk) {
+    const uint64_t steps = (uint64_t)B * (uint64_t)(A.T > 0 ? A.T : 1);
+    const uint64_t k_step = (uint64_t)A.Hk * Dk, v_step = (uint64_t)A.Hv * A.Dv, C = 2 * k_step + v_step;
+    if (A.Hv > 65535 || B > 65535 || C >= (1u << 24) || steps * k_step >= (1ull << 31) || steps * v_step >= (1ull << 31)) return false;
+    A.group = (uint32_t)(A.Hv / A.Hk);
+    A.group_magic = A.group > 1 ? (uint32_t)(((1ull << 32) + A.group - 1) / A.group) : 0u;
+    return true;
+}
+
 template <int DK>
 static int launch_gdn_layer(hipStream_t st, const GdnArgs& A, const GdnPrep& P, int B) {
     const size_t lds = sizeof(GdnChunkLds<DK>);
-    dim3 grid(A.Dv / kChunkRows, B * A.Hv);
+    dim3 grid(A.Dv / kChunkRows, A.Hv, B);
     LaunchBracket br(DFLASH_KERNEL_GDN_LAYER, st);
     br.launch(gdn_layer_kernel<DK>, grid, dim3(kThreads), lds, A, P);
     DFLASH_HIP_TRY(hipGetLastError());
@@ -1171,7 +1192,7 @@ static int launch_gdn_layer(hipStream_t st, const GdnArgs& A, const GdnPrep& P, 
 template <int DK>
 static int launch_gdn_chunk(hipStream_t st, const GdnArgs& A, int B) {
     const size_t lds = sizeof(GdnChunkLds<DK>);     // the attribute that allows it is set per device by gdn_device_setup()
-    dim3 grid(A.Dv / kChunkRows, B * A.Hv);
+    dim3 grid(A.Dv / kChunkRows, A.Hv, B);
     LaunchBracket br(DFLASH_KERNEL_GDN_FORWARD, st);
     if (A.mask) br.launch(gated_delta_chunk_kernel<true, DK>, grid, dim3(kThreads), lds, A);
     else br.launch(gated_delta_chunk_kernel<false, DK>, grid, dim3(kThreads), lds, A);
@@ -1288,7 +1309,7 @@ extern "C" int dflash_gated_delta_tape(void* stream, const void* q, const void* 
     A.q = q; A.k = k; A.v = v; A.g = g; A.beta = beta; A.mask = mask;
     A.state_in = state_in; A.state_out = state_out; A.y = y; A.tape = tape_out;
     A.in_dtype = in_dtype; A.mask_dtype = mask_dtype; A.T = T; A.Hk = Hk; A.Hv = Hv; A.Dv = Dv;
-    if (state_dtype == DFLASH_F32 && g_ndim == 3 && Dv % kChunkRows == 0 && T > 0) {
+    if (state_dtype == DFLASH_F32 && g_ndim == 3 && Dv % kChunkRows == 0 && T > 0 && chunk_index_setup(A, B, Dk)) {
         // fp32 state with one decay per head and step: chunked form
         if (Dk == 64) return launch_gdn_chunk<64>((hipStream_t)stream, A, B);
         if (Dk == 128) return launch_gdn_chunk<128>((hipStream_t)stream, A, B);
@@ -1329,6 +1350,7 @@ extern "C" int dflash_gdn_layer(void* stream, const void* mixed_qkv, const void*
     A.q = A.k = A.v = A.g = A.beta = A.mask = nullptr;
     A.state_in = state_in; A.state_out = state_out; A.y = y_out; A.tape = tape_out;
     A.in_dtype = in_dtype; A.mask_dtype = 0; A.T = T; A.Hk = Hk; A.Hv = Hv; A.Dv = Dv;
+    DFLASH_SUPPORTED(chunk_index_setup(A, B, Dk), "gdn_layer: shape beyond the chunked kernel's 32-bit element offsets");
     GdnPrep P;
     P.x = mixed_qkv; P.conv_in = conv_state_in; P.weight = conv_weight; P.a = a_logits; P.b = b_logits;
     P.a_log = a_log; P.dt_bias = dt_bias; P.q_out = q_out; P.k_out = k_out; P.v_out = v_out; P.g_out = g_out;
