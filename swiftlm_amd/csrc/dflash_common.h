@@ -80,6 +80,16 @@ inline int dtype_size(int dt) {
     }
 }
 
+// n / d by one multiply: magic = floor(2^32 / d) (as close as 32 bits allow for d == 1) gives a quotient that is
+// at most one too small for any n < 2^32; one comparison corrects it.  An integer division by a run-time value is
+// some twenty-five dependent instructions, which matters ahead of a kernel's first load.
+inline uint32_t fast_div_magic(uint32_t d) { return d <= 1 ? 0xFFFFFFFFu : (uint32_t)((1ull << 32) / d); }
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t d, uint32_t magic) {
+    uint32_t q = __umulhi(n, magic);
+    q += (n - q * d) >= d;
+    return q;
+}
+
 // ---- element types -------------------------------------------------------
 
 struct bf16_t { uint16_t bits; };

@@ -99,6 +99,7 @@ struct SdpaArgs {
     const int32_t* page_table;
     int page_shift, table_stride, num_pages;
     int32_t* status;         // device status word (dflash_set_status_word), or null
+    uint32_t gpk_magic, S_magic;   // fast_div_magic of groups_per_kv and S
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -225,7 +226,7 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
                  "s"(A.part_m), "s"(A.part_l), "s"(A.kv_len_dev), "s"(A.mask), "s"(A.kv_batch_stride), "s"(A.kv_head_stride));
     asm volatile("" ::"s"(A.scale_log2), "s"(A.Hq), "s"(A.Hk), "s"(A.G), "s"(A.N), "s"(A.S), "s"(A.groups_per_kv),
                  "s"(A.rows_total), "s"(A.len_bias), "s"(A.page_table), "s"(A.page_shift), "s"(A.table_stride), "s"(A.num_pages),
-                 "s"(A.status));
+                 "s"(A.status), "s"(A.gpk_magic), "s"(A.S_magic));
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -233,8 +234,8 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
     const bool producer = wave >= 4;
     const int c = lane & 31, h = lane >> 5;
     const int split = blockIdx.x;
-    const int hk = blockIdx.y / A.groups_per_kv;
-    const int hg0 = (blockIdx.y % A.groups_per_kv) * kHeadsPerWG;
+    const int hk = (int)fast_div(blockIdx.y, (uint32_t)A.groups_per_kv, A.gpk_magic);
+    const int hg0 = ((int)blockIdx.y - hk * A.groups_per_kv) * kHeadsPerWG;
     const int b = blockIdx.z;
     const int hcount = (A.G - hg0) < kHeadsPerWG ? (A.G - hg0) : kHeadsPerWG;
 
@@ -292,21 +293,8 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
             }
         }
     }
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(len_raw));
-    int Nb = A.kv_len_dev ? len_raw + A.len_bias : A.N;
-    if (A.status && (Nb < kM || Nb > A.N) && split == 0 && blockIdx.y == 0 && tid == 0) atomicOr(A.status, DFLASH_STATUS_SDPA_LEN);
-    Nb = Nb < kM ? kM : (Nb > A.N ? A.N : Nb);
-    const int nt = (Nb + kBN - 1) / kBN;
-    // Tiles are dealt round-robin: split s takes tiles s, s + S, s + 2S, ...  At any moment the workgroups of a KV
-    // head then read one contiguous stretch of the cache (S neighbouring tiles) instead of S stretches a split
-    // apart, which the memory system serves faster.  Below, t counts this split's own tiles (0 .. t_end-1) and
-    // key_of(t) is the first key of its t-th tile.
-    const int t_begin = 0;
-    const int t_full = nt / A.S;                                   // rows of S tiles that every split takes part in
-    const int t_end = t_full + (tile_index(split, t_full, A.S) < nt ? 1 : 0);
-    const int t_last = t_end - 1;
-    auto key_of = [&](int t) { return tile_index(split, t, A.S) * kBN; };
-
+    // Everything that does not depend on the key count is worked out while the count is on its way (the bases are
+    // operands of the wait below, so that they are in registers before it, not behind it).
     const int cw = producer ? 0 : wave;                      // compute wave index (producers: unused)
     const int head_in_group = 2 * cw + (c >> 4);
     const bool row_valid = !producer && head_in_group < hcount;
@@ -320,6 +308,23 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
                                   : ((size_t)b * A.kv_batch_stride + (size_t)hk * A.kv_head_stride) * 2;
     const unsigned char* kbase = reinterpret_cast<const unsigned char*>(A.k) + head_off;
     const unsigned char* vbase = reinterpret_cast<const unsigned char*>(A.v) + head_off;
+    const unsigned char* knew = reinterpret_cast<const unsigned char*>(A.k_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
+    const unsigned char* vnew = reinterpret_cast<const unsigned char*>(A.v_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(len_raw) : "s"(kbase), "s"(vbase), "s"(knew), "s"(vnew));
+    int Nb = A.kv_len_dev ? len_raw + A.len_bias : A.N;
+    if (A.status && (Nb < kM || Nb > A.N) && split == 0 && blockIdx.y == 0 && tid == 0) atomicOr(A.status, DFLASH_STATUS_SDPA_LEN);
+    Nb = Nb < kM ? kM : (Nb > A.N ? A.N : Nb);
+    const int nt = (Nb + kBN - 1) / kBN;
+    // Tiles are dealt round-robin: split s takes tiles s, s + S, s + 2S, ...  At any moment the workgroups of a KV
+    // head then read one contiguous stretch of the cache (S neighbouring tiles) instead of S stretches a split
+    // apart, which the memory system serves faster.  Below, t counts this split's own tiles (0 .. t_end-1) and
+    // key_of(t) is the first key of its t-th tile.
+    const int t_begin = 0;
+    const int t_full = (int)fast_div((uint32_t)nt, (uint32_t)A.S, A.S_magic);    // rows of S tiles that every split takes part in
+    const int t_end = t_full + (tile_index(split, t_full, A.S) < nt ? 1 : 0);
+    const int t_last = t_end - 1;
+    auto key_of = [&](int t) { return tile_index(split, t, A.S) * kBN; };
+
     // Byte offset of key n's row from kbase / vbase (the K and V pools share one layout), for the rows that are
     // looked up one by one: those of the fused append.  Paged: the page comes from the table, clamped to the pool.
     // (Tiles take tile_off() below; a tile never straddles a page, page sizes being multiples of kBN.)
@@ -339,8 +344,6 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
     // in that workgroup, which then finished last of the launch).
     const bool fused = A.k_new != nullptr;
     const int cache_rows = fused ? Nb - kM : Nb;       // keys below this index are read from the cache
-    const unsigned char* knew = reinterpret_cast<const unsigned char*>(A.k_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
-    const unsigned char* vnew = reinterpret_cast<const unsigned char*>(A.v_new) + ((size_t)b * A.Hk + hk) * kM * L::ROWB;
     if (fused && A.k_cache && hg0 == 0 && wave == 0) {
         // 16-byte pieces of the block's rows, dealt evenly over the splits of the KV head: a handful per workgroup,
         // read and written by the first compute wave in one round trip.
@@ -1039,6 +1042,7 @@ static int sdpa_common(void* stream, const void* q, const void* k, const void* v
     A.kv_batch_stride = kv_batch_stride; A.kv_head_stride = kv_head_stride;
     A.scale_log2 = scale * 1.4426950408889634f;
     A.Hq = Hq; A.Hk = Hk; A.G = G; A.N = N; A.S = S; A.groups_per_kv = groups; A.rows_total = B * Hq * kM;
+    A.gpk_magic = fast_div_magic((uint32_t)groups); A.S_magic = fast_div_magic((uint32_t)S);
     A.len_bias = k_new ? kM : 0;
     A.page_table = paged ? paged->table : nullptr;
     A.page_shift = page_shift;
