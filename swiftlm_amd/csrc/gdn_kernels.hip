@@ -627,7 +627,42 @@ template <int DK> struct GdnChunkLds {
     float v[16][16];                       // v_t of row r at v[t][r]
     float g[16], beta[16], gam[16], w[16]; // w[s] = G[s][15]: decay from step s to the end of the chunk
     int on[16];
+    // bf16 inputs: the product's operands as bf16 (x rows 16..31 and y rows 16..31 are then unused).  The state tile
+    // as three bf16 terms, S_0 = hi + mid + lo exactly (3 x 8 = 24 significand bits); k_t and q_t as they came.
+    // Row pitch DK + 8: the 16 bytes of pad spread a column of rows over all banks for 16-byte reads.
+    static constexpr int LB = DK + 8;
+    uint16_t xs[3][16][LB];
+    uint16_t kb[16][LB], qb[16][LB];
 };
+
+typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
+
+// Four floats that are bf16 values -> their 4 x 16 bits.
+__device__ __forceinline__ uint2 pack4_bf16_exact(float4 v) {
+    uint2 u;
+    u.x = (__float_as_uint(v.x) >> 16) | (__float_as_uint(v.y) & 0xffff0000u);
+    u.y = (__float_as_uint(v.z) >> 16) | (__float_as_uint(v.w) & 0xffff0000u);
+    return u;
+}
+// x = hi + mid + lo with each term a bf16: hi = bf16(x), mid = bf16(x - hi), lo = x - hi - mid (8 bits are left, so
+// lo is exact and the three add up to x bit for bit; both subtractions are exact as well).
+__device__ __forceinline__ void split3_bf16(float x, uint16_t& hi, uint16_t& mid, uint16_t& lo) {
+    hi = f32_to_bf16_bits(x);
+    const float r1 = x - __uint_as_float((uint32_t)hi << 16);
+    mid = f32_to_bf16_bits(r1);
+    const float r2 = r1 - __uint_as_float((uint32_t)mid << 16);
+    lo = f32_to_bf16_bits(r2);
+}
+__device__ __forceinline__ void split3_bf16(float4 v, uint2& hi, uint2& mid, uint2& lo) {
+    uint16_t h[4], m[4], l[4];
+    split3_bf16(v.x, h[0], m[0], l[0]);
+    split3_bf16(v.y, h[1], m[1], l[1]);
+    split3_bf16(v.z, h[2], m[2], l[2]);
+    split3_bf16(v.w, h[3], m[3], l[3]);
+    hi = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
+    mid = make_uint2(m[0] | ((uint32_t)m[1] << 16), m[2] | ((uint32_t)m[3] << 16));
+    lo = make_uint2(l[0] | ((uint32_t)l[1] << 16), l[2] | ((uint32_t)l[3] << 16));
+}
 
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 typedef float f32x16v __attribute__((ext_vector_type(16)));
@@ -653,7 +688,8 @@ template <int S> struct SolveStep {
     }
 };
 
-template <bool HAS_MASK, int DK, bool FUSED>
+// BF: the inputs are bf16 (fixed at compile time): the product then runs on bf16 MFMAs, exactly (see below).
+template <bool HAS_MASK, int DK, bool FUSED, bool BF>
 __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& P) {
     using Lds = GdnChunkLds<DK>;
     extern __shared__ __align__(16) unsigned char gdn_chunk_smem[];
@@ -708,6 +744,29 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         sv0[u] = load4(s_in + (uint32_t)(r * DK + c4));
     }
 
+    // Where the staged operands go: fp32 rows for the fp32 product (x = [S_0 ; k], y = [k ; q]); with bf16 inputs the
+    // product reads the bf16 arrays instead, and only what the state update needs stays fp32 (S_0 and k).
+    auto store_state4 = [&](int r, int c4, float4 s4) {
+        store4(&L.x[r][c4], s4);
+        if constexpr (BF) {
+            uint2 hi, mid, lo;
+            split3_bf16(s4, hi, mid, lo);
+            *reinterpret_cast<uint2*>(&L.xs[0][r][c4]) = hi;
+            *reinterpret_cast<uint2*>(&L.xs[1][r][c4]) = mid;
+            *reinterpret_cast<uint2*>(&L.xs[2][r][c4]) = lo;
+        }
+    };
+    auto store_kq4 = [&](int t, int c4, float4 k4, float4 q4) {
+        store4(&L.y[t][c4], k4);
+        if constexpr (BF) {
+            *reinterpret_cast<uint2*>(&L.kb[t][c4]) = pack4_bf16_exact(k4);
+            *reinterpret_cast<uint2*>(&L.qb[t][c4]) = pack4_bf16_exact(q4);
+        } else {
+            store4(&L.x[16 + t][c4], k4);
+            store4(&L.y[16 + t][c4], q4);
+        }
+    };
+
     // Stage one chunk: every global load of the chunk (the state tile is already on its way) is issued
     // before the first conversion or LDS store, so the chunk pays one memory round trip, not one per array.
     // Steps >= tc are identity steps.  Elem is the element type of q/k/v/g/beta.
@@ -746,16 +805,13 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
 #pragma unroll
             for (int u = 0; u < NV; ++u) {
                 const int i = tid + u * kThreads, r = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
-                store4(&L.x[r][c4], sv0[u]);
+                store_state4(r, c4, sv0[u]);
             }
         }
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
             const int i = tid + u * kThreads, t = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
-            const float4 k4 = t < tc ? kv[u] : zero4, q4 = t < tc ? qv[u] : zero4;
-            store4(&L.x[16 + t][c4], k4);
-            store4(&L.y[t][c4], k4);
-            store4(&L.y[16 + t][c4], q4);
+            store_kq4(t, c4, t < tc ? kv[u] : zero4, t < tc ? qv[u] : zero4);
         }
         L.v[ts][tt] = ts < tc ? vv : 0.f;
         if (tid < kChunkSteps) {
@@ -822,7 +878,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
             const int i = tid + u * kThreads, r = i / (DK / 4), cc = (i % (DK / 4)) * 4;
-            store4(&L.x[r][cc], sv0[u]);
+            store_state4(r, cc, sv0[u]);
         }
         const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
         const bool first_tile = blockIdx.x == 0;
@@ -857,9 +913,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
             const float4 kc = conv4(kw[u], ktap, tl), qc = conv4(qw[u], qtap, tl);
             const float4 k4 = round4(kc, head_scale(kc, P.k_scale)), q4 = round4(qc, head_scale(qc, P.q_scale));
             const bool live = t < tc;
-            store4(&L.x[16 + t][c4], live ? k4 : zero4);
-            store4(&L.y[t][c4], live ? k4 : zero4);
-            store4(&L.y[16 + t][c4], live ? q4 : zero4);
+            store_kq4(t, c4, live ? k4 : zero4, live ? q4 : zero4);
             if (qk_owner && live) {
                 const size_t o = (((size_t)b * A.T + t) * A.Hk + hk) * DK + c4;
                 if (P.k_out) store4(reinterpret_cast<Elem*>(P.k_out) + o, k4);
@@ -948,11 +1002,11 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         const int tc = (A.T - t0) < kChunkSteps ? (A.T - t0) : kChunkSteps;
         const bool last_chunk = t0 + kChunkSteps >= A.T;
         if constexpr (FUSED) {
-            if (A.in_dtype == DFLASH_BF16) stage_fused(bf16_t{}, tc);
+            if constexpr (BF) stage_fused(bf16_t{}, tc);
             else if (A.in_dtype == DFLASH_F16) stage_fused(f16_t{}, tc);
             else stage_fused(float{}, tc);
         } else {
-            if (A.in_dtype == DFLASH_BF16) stage(bf16_t{}, t0, tc, t0 == 0);
+            if constexpr (BF) stage(bf16_t{}, t0, tc, t0 == 0);
             else if (A.in_dtype == DFLASH_F16) stage(f16_t{}, t0, tc, t0 == 0);
             else stage(float{}, t0, tc, t0 == 0);
         }
@@ -966,14 +1020,34 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         {
             const int n = lane % 16, kk = lane / 16;
             const int ws = __builtin_amdgcn_readfirstlane(w);
-            const float* ap = &L.x[(ws < 2 ? 0 : 16) + n][4 * kk];
-            const float* bp = &L.y[(ws & 1 ? 16 : 0) + n][4 * kk];
-            constexpr int NB = DK / 16, PS = 4 * NB / 16;     // 4*NB MFMAs, 15 pieces
-            float4 av[NB], bv[NB];
+            constexpr int NB = DK / 16, PS = 4 * NB / 16;     // fp32 product: 4*NB MFMAs, 15 pieces
+            constexpr int NK = DK / 32;                       // bf16 product: contraction steps of 32 channels
+            float4 av[BF ? 1 : NB], bv[BF ? 1 : NB];
+            bf16x8v ah[BF ? NK : 1], am[BF ? NK : 1], al[BF ? NK : 1], bb[BF ? NK : 1];
+            if constexpr (BF) {
+                // A 16x16x32 bf16 MFMA takes lane l's a as row l%16, channels 8*(l/16) .. +7 of the step (b alike).
+                const uint16_t* bq = (ws & 1) ? &L.qb[n][8 * kk] : &L.kb[n][8 * kk];
+                const int arow = ws < 2 ? 0 : 1;              // waves 2, 3 take k rows as their a operand
 #pragma unroll
-            for (int c = 0; c < NB; ++c) {
-                av[c] = *reinterpret_cast<const float4*>(ap + 16 * c);
-                bv[c] = *reinterpret_cast<const float4*>(bp + 16 * c);
+                for (int ks = 0; ks < NK; ++ks) {
+                    bb[ks] = *reinterpret_cast<const bf16x8v*>(bq + 32 * ks);
+                    ah[ks] = *reinterpret_cast<const bf16x8v*>((arow ? &L.kb[n][8 * kk] : &L.xs[0][n][8 * kk]) + 32 * ks);
+                }
+                if (ws < 2) {
+#pragma unroll
+                    for (int ks = 0; ks < NK; ++ks) {
+                        am[ks] = *reinterpret_cast<const bf16x8v*>(&L.xs[1][n][8 * kk + 32 * ks]);
+                        al[ks] = *reinterpret_cast<const bf16x8v*>(&L.xs[2][n][8 * kk + 32 * ks]);
+                    }
+                }
+            } else {
+                const float* ap = &L.x[(ws < 2 ? 0 : 16) + n][4 * kk];
+                const float* bp = &L.y[(ws & 1 ? 16 : 0) + n][4 * kk];
+#pragma unroll
+                for (int c = 0; c < NB; ++c) {
+                    av[c] = *reinterpret_cast<const float4*>(ap + 16 * c);
+                    bv[c] = *reinterpret_cast<const float4*>(bp + 16 * c);
+                }
             }
             float gj[kChunkSteps];
 #pragma unroll
@@ -1017,6 +1091,34 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
             };
             f32x4v acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
             __builtin_amdgcn_sched_barrier(0);
+            if constexpr (BF) {
+                // With bf16 inputs the same product is exact on bf16 MFMAs: k and q are bf16, and the fp32 state
+                // enters as three bf16 terms that add up to it bit for bit, so every partial product is exact in
+                // fp32 and only the order of the additions differs from the fp32 MFMA.  3*NK MFMAs of 8 passes for
+                // the state blocks, NK for the k blocks (whose waves also form the decay products), against 4*NB of
+                // 8 passes in fp32.
+                if (ws < 2) {
+#pragma unroll
+                    for (int ks = 0; ks < NK; ++ks) {
+                        acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah[ks], bb[ks], acc0, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am[ks], bb[ks], acc1, 0, 0, 0);
+                        acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al[ks], bb[ks], acc0, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) coef[v] = 1.f;
+                } else {
+                    constexpr int PP = 16 / NK;         // pieces behind each MFMA
+#pragma unroll
+                    for (int ks = 0; ks < NK; ++ks) {
+                        if (ks & 1) acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah[ks], bb[ks], acc1, 0, 0, 0);
+                        else acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah[ks], bb[ks], acc0, 0, 0, 0);
+#pragma unroll
+                        for (int pc = 0; pc < PP; ++pc) g_piece(ks * PP + pc);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+            if constexpr (!BF)
 #pragma unroll
             for (int c = 0; c < NB; c += 2) {
                 const float a0[4] = {av[c].x, av[c].y, av[c].z, av[c].w}, b0[4] = {bv[c].x, bv[c].y, bv[c].z, bv[c].w};
@@ -1126,7 +1228,11 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
 #pragma unroll
-                    for (int e = 0; e < E; ++e) L.x[4 * kk + v][base + e] = cacc[e][v];
+                    for (int e = 0; e < E; ++e) {
+                        L.x[4 * kk + v][base + e] = cacc[e][v];
+                        if constexpr (BF) split3_bf16(cacc[e][v], L.xs[0][4 * kk + v][base + e], L.xs[1][4 * kk + v][base + e],
+                                                      L.xs[2][4 * kk + v][base + e]);
+                    }
                     asm volatile("" ::: "memory");
                 }
                 // the staging barrier of the next chunk orders these writes before their readers
@@ -1157,15 +1263,15 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         for (int t0 = kChunkSteps; t0 < A.T; t0 += kChunkSteps) run_chunk(t0);
 }
 
-template <bool HAS_MASK, int DK>
+template <bool HAS_MASK, int DK, bool BF>
 __global__ __launch_bounds__(kThreads) void gated_delta_chunk_kernel(GdnArgs A) {
-    gdn_chunk_body<HAS_MASK, DK, false>(A, GdnPrep{});
+    gdn_chunk_body<HAS_MASK, DK, false, BF>(A, GdnPrep{});
 }
 
 // One GatedDelta layer from its projections to the recurrence's outputs in one launch.
-template <int DK>
+template <int DK, bool BF>
 __global__ __launch_bounds__(kThreads) void gdn_layer_kernel(GdnArgs A, GdnPrep P) {
-    gdn_chunk_body<false, DK, true>(A, P);
+    gdn_chunk_body<false, DK, true, BF>(A, P);
 }
 
 // Whether the chunked kernels' 32-bit element offsets and 24-bit per-step strides cover this shape, and the
@@ -1184,7 +1290,8 @@ static int launch_gdn_layer(hipStream_t st, const GdnArgs& A, const GdnPrep& P, 
     const size_t lds = sizeof(GdnChunkLds<DK>);
     dim3 grid(A.Dv / kChunkRows, A.Hv, B);
     LaunchBracket br(DFLASH_KERNEL_GDN_LAYER, st);
-    br.launch(gdn_layer_kernel<DK>, grid, dim3(kThreads), lds, A, P);
+    if (A.in_dtype == DFLASH_BF16) br.launch(gdn_layer_kernel<DK, true>, grid, dim3(kThreads), lds, A, P);
+    else br.launch(gdn_layer_kernel<DK, false>, grid, dim3(kThreads), lds, A, P);
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
 }
@@ -1194,8 +1301,11 @@ static int launch_gdn_chunk(hipStream_t st, const GdnArgs& A, int B) {
     const size_t lds = sizeof(GdnChunkLds<DK>);     // the attribute that allows it is set per device by gdn_device_setup()
     dim3 grid(A.Dv / kChunkRows, A.Hv, B);
     LaunchBracket br(DFLASH_KERNEL_GDN_FORWARD, st);
-    if (A.mask) br.launch(gated_delta_chunk_kernel<true, DK>, grid, dim3(kThreads), lds, A);
-    else br.launch(gated_delta_chunk_kernel<false, DK>, grid, dim3(kThreads), lds, A);
+    const bool bf = A.in_dtype == DFLASH_BF16;
+    if (A.mask && bf) br.launch(gated_delta_chunk_kernel<true, DK, true>, grid, dim3(kThreads), lds, A);
+    else if (A.mask) br.launch(gated_delta_chunk_kernel<true, DK, false>, grid, dim3(kThreads), lds, A);
+    else if (bf) br.launch(gated_delta_chunk_kernel<false, DK, true>, grid, dim3(kThreads), lds, A);
+    else br.launch(gated_delta_chunk_kernel<false, DK, false>, grid, dim3(kThreads), lds, A);
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
 }
@@ -1203,9 +1313,12 @@ static int launch_gdn_chunk(hipStream_t st, const GdnArgs& A, int B) {
 template <int DK>
 static int gdn_chunk_setup() {
     const int lds = (int)sizeof(GdnChunkLds<DK>);
-    DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<true, DK>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<false, DK>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gdn_layer_kernel<DK>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<true, DK, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<true, DK, false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<false, DK, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<false, DK, false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gdn_layer_kernel<DK, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    DFLASH_HIP_TRY(hipFuncSetAttribute((const void*)gdn_layer_kernel<DK, false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     return DFLASH_OK;
 }
 

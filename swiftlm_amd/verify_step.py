@@ -215,7 +215,8 @@ class HybridVerifyStack:
         cfg, T = self.cfg, self.cfg.block
         assert cfg.Dk in (64, 128, 256) and cfg.Dv % 16 == 0 and cfg.Hq // cfg.Hkv <= 8 and cfg.D in (128, 256)
         ld = cfg.Dk + 4
-        gdn_lds = 4 * (2 * 32 * ld + 4 * 32 * 33 + 32 * 33 + 2 * 16 * 16 + 16 * 17 + 16 * 16 + 4 * 16 + 16)
+        gdn_lds = (4 * (2 * 32 * ld + 16 * 33 + 2 * 16 * 16 + 16 * 17 + 16 * 16 + 4 * 16 + 16)   # fp32 operands and tables
+                   + 2 * 5 * 16 * (cfg.Dk + 8))                                                    # bf16 operands
         gdn = (cfg.Dv // 16, cfg.Hv, 1, 256, gdn_lds)
         # splits: the S whose workspace layout gives the size the library reports
         rows = cfg.Hq * T
