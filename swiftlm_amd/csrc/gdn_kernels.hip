@@ -637,31 +637,33 @@ template <int DK> struct GdnChunkLds {
 
 typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
 
+// The upper halves of two words as one: (a >> 16) | (b & 0xffff0000), one v_perm_b32.
+__device__ __forceinline__ uint32_t upper_halves(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
 // Four floats that are bf16 values -> their 4 x 16 bits.
 __device__ __forceinline__ uint2 pack4_bf16_exact(float4 v) {
-    uint2 u;
-    u.x = (__float_as_uint(v.x) >> 16) | (__float_as_uint(v.y) & 0xffff0000u);
-    u.y = (__float_as_uint(v.z) >> 16) | (__float_as_uint(v.w) & 0xffff0000u);
-    return u;
+    return make_uint2(upper_halves(__float_as_uint(v.x), __float_as_uint(v.y)), upper_halves(__float_as_uint(v.z), __float_as_uint(v.w)));
 }
-// x = hi + mid + lo with each term a bf16: hi = bf16(x), mid = bf16(x - hi), lo = x - hi - mid (8 bits are left, so
-// lo is exact and the three add up to x bit for bit; both subtractions are exact as well).
+// x = hi + mid + lo with each term a bf16, by truncation: hi = the upper 16 bits of x, mid = the upper 16 bits of
+// x - hi, lo = x - hi - mid.  hi takes 8 of x's 24 significand bits, mid the next 8 (or more, where zeros follow hi),
+// so lo has at most 8 left and is a bf16 as it stands; both subtractions are exact, and the three terms add up to x
+// bit for bit.  Four VALU operations per value and one v_perm per pair and term.
+__device__ __forceinline__ void split3_bf16(float x, float& r1, float& r2) {
+    r1 = x - __uint_as_float(__float_as_uint(x) & 0xffff0000u);
+    r2 = r1 - __uint_as_float(__float_as_uint(r1) & 0xffff0000u);
+}
 __device__ __forceinline__ void split3_bf16(float x, uint16_t& hi, uint16_t& mid, uint16_t& lo) {
-    hi = f32_to_bf16_bits(x);
-    const float r1 = x - __uint_as_float((uint32_t)hi << 16);
-    mid = f32_to_bf16_bits(r1);
-    const float r2 = r1 - __uint_as_float((uint32_t)mid << 16);
-    lo = f32_to_bf16_bits(r2);
+    float r1, r2;
+    split3_bf16(x, r1, r2);
+    hi = (uint16_t)(__float_as_uint(x) >> 16); mid = (uint16_t)(__float_as_uint(r1) >> 16); lo = (uint16_t)(__float_as_uint(r2) >> 16);
 }
 __device__ __forceinline__ void split3_bf16(float4 v, uint2& hi, uint2& mid, uint2& lo) {
-    uint16_t h[4], m[4], l[4];
-    split3_bf16(v.x, h[0], m[0], l[0]);
-    split3_bf16(v.y, h[1], m[1], l[1]);
-    split3_bf16(v.z, h[2], m[2], l[2]);
-    split3_bf16(v.w, h[3], m[3], l[3]);
-    hi = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
-    mid = make_uint2(m[0] | ((uint32_t)m[1] << 16), m[2] | ((uint32_t)m[3] << 16));
-    lo = make_uint2(l[0] | ((uint32_t)l[1] << 16), l[2] | ((uint32_t)l[3] << 16));
+    const float x[4] = {v.x, v.y, v.z, v.w};
+    float r1[4], r2[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) split3_bf16(x[i], r1[i], r2[i]);
+    hi = make_uint2(upper_halves(__float_as_uint(x[0]), __float_as_uint(x[1])), upper_halves(__float_as_uint(x[2]), __float_as_uint(x[3])));
+    mid = make_uint2(upper_halves(__float_as_uint(r1[0]), __float_as_uint(r1[1])), upper_halves(__float_as_uint(r1[2]), __float_as_uint(r1[3])));
+    lo = make_uint2(upper_halves(__float_as_uint(r2[0]), __float_as_uint(r2[1])), upper_halves(__float_as_uint(r2[2]), __float_as_uint(r2[3])));
 }
 
 typedef float f32x4v __attribute__((ext_vector_type(4)));
@@ -1177,9 +1179,11 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
             yv = L.on[t] ? yv : 0.f;
             if (t < tc) {
                 const uint32_t o = (((uint32_t)b * A.T + t0) * A.Hv + hv) * A.Dv + row0 + __umul24(t, v_step) + r;
-                if (FUSED && P.fin_gate) store1_rt_agent(A.y, A.in_dtype, o, yv);   // re-read by the head's last workgroup
-                else store1_rt(A.y, A.in_dtype, o, yv);
-                A.tape[o] = L.dl[t][r];
+                // Written through (agent scope): the 32- and 64-byte pieces then leave the L2s as they are produced
+                // instead of waiting as partly dirty lines for the end-of-launch flush; the layer kernel's last
+                // workgroup of a head re-reads y at that scope.
+                store1_rt_agent(A.y, A.in_dtype, o, yv);
+                __hip_atomic_store(A.tape + o, L.dl[t][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             if constexpr (FUSED) {
                 if (P.fin_gate) {          // this tile's share of sum(y^2) of step t, parked in the row of `out`
