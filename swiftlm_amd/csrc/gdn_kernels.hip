@@ -780,6 +780,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         const Elem* gp = reinterpret_cast<const Elem*>(A.g);
         const Elem* bp = reinterpret_cast<const Elem*>(A.beta);
         float4 kv[NV], qv[NV];
+        uint2 kraw[NV], qraw[NV];               // bf16 inputs: the rows as they come (q is never widened)
         const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
         const uint32_t bt0 = (uint32_t)b * A.T + t0;                       // first step of the chunk, all uniform
         const uint32_t k0 = (bt0 * A.Hk + hk) * DK, v0 = (bt0 * A.Hv + hv) * A.Dv + row0, g0 = bt0 * A.Hv + hv;
@@ -788,8 +789,13 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
             const int i = tid + u * kThreads, t = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
             const int tl = t < tc ? t : tc - 1;           // clamped: always a valid address, selected away below
             const uint32_t o = k0 + __umul24(tl, k_step) + c4;
-            kv[u] = load4(kp + o);
-            qv[u] = load4(qp + o);
+            if constexpr (BF) {
+                kraw[u] = *reinterpret_cast<const uint2*>(kp + o);
+                qraw[u] = *reinterpret_cast<const uint2*>(qp + o);
+            } else {
+                kv[u] = load4(kp + o);
+                qv[u] = load4(qp + o);
+            }
         }
         const int tvl = ts < tc ? ts : tc - 1;
         const float vv = to_float(vp[v0 + __umul24(tvl, v_step) + tt]);
@@ -813,7 +819,15 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
             const int i = tid + u * kThreads, t = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
-            store_kq4(t, c4, t < tc ? kv[u] : zero4, t < tc ? qv[u] : zero4);
+            if constexpr (BF) {
+                const uint2 kr = t < tc ? kraw[u] : make_uint2(0u, 0u), qr = t < tc ? qraw[u] : make_uint2(0u, 0u);
+                store4(&L.y[t][c4], make_float4(__uint_as_float(kr.x << 16), __uint_as_float(kr.x & 0xffff0000u),
+                                                __uint_as_float(kr.y << 16), __uint_as_float(kr.y & 0xffff0000u)));
+                *reinterpret_cast<uint2*>(&L.kb[t][c4]) = kr;
+                *reinterpret_cast<uint2*>(&L.qb[t][c4]) = qr;
+            } else {
+                store_kq4(t, c4, t < tc ? kv[u] : zero4, t < tc ? qv[u] : zero4);
+            }
         }
         L.v[ts][tt] = ts < tc ? vv : 0.f;
         if (tid < kChunkSteps) {
