@@ -335,8 +335,9 @@ def test_gdn_finish_matches_oracle(gpu_lib, shape, in_dt, kind):
 # ---- one-launch layer: pre-ops inside the forward kernel (KimiLinearDFlash.swift:351-378) ----
 
 @pytest.mark.parametrize("cfg", [(1, 16, 16, 32, 128, 128), (2, 5, 2, 4, 64, 48), (1, 2, 1, 2, 256, 32),
-                                 (1, 1, 2, 2, 128, 16), (1, 16, 4, 8, 64, 64)],
-                         ids=["qwen3next_block", "short_block_b2", "T_shorter_than_window_dk256", "single_step", "dk64"])
+                                 (1, 1, 2, 2, 128, 16), (1, 16, 4, 8, 64, 64), (2, 7, 2, 6, 128, 32)],
+                         ids=["qwen3next_block", "short_block_b2", "T_shorter_than_window_dk256", "single_step", "dk64",
+                              "three_value_heads_per_key_head_b2"])
 @pytest.mark.parametrize("in_dt", ["bf16", "f32", "f16"])
 @pytest.mark.parametrize("carry", [True, False], ids=["conv_state", "no_conv_state"])
 def test_gdn_layer_equals_prepare_forward_finish_bitwise(gpu_lib, cfg, in_dt, carry):
