@@ -671,7 +671,7 @@ typedef float f32x16v __attribute__((ext_vector_type(16)));
 
 template <int QUAD_LANE> __device__ __forceinline__ float quad_broadcast(float x) {
     constexpr int ctrl = QUAD_LANE | (QUAD_LANE << 2) | (QUAD_LANE << 4) | (QUAD_LANE << 6);
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), ctrl, 0xf, 0xf, false));
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), ctrl, 0xf, 0xf, true));
 }
 
 // Steps S..15 of the unit-triangular solve for one state row held by a quad (lane q owns steps 4q..4q+3).
@@ -1171,13 +1171,19 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
             const int r = lane / 4, q = lane % 4;
             float acc[4], bet[16], mine[4] = {0.f, 0.f, 0.f, 0.f};
             float4 arow[16];
+            // every LDS read of the phase goes out before the first use (the compiler keeps the order written here:
+            // with the start values first, the coefficient reads waited for them -- a second trip to LDS)
+            float gm[4], pv[4], vv[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc[e] = fmaf(-L.gam[4 * q + e], L.p[r][4 * q + e], L.v[4 * q + e][r]);
+            for (int e = 0; e < 4; ++e) { gm[e] = L.gam[4 * q + e]; pv[e] = L.p[r][4 * q + e]; vv[e] = L.v[4 * q + e][r]; }
 #pragma unroll
             for (int s = 0; s < 16; ++s) {
                 arow[s] = *reinterpret_cast<const float4*>(&L.a[s][4 * q]);
                 bet[s] = L.beta[s];
             }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] = fmaf(-gm[e], pv[e], vv[e]);
             SolveStep<0>::run(acc, arow, bet, mine, q);
 #pragma unroll
             for (int e = 0; e < 4; ++e) L.dl[4 * q + e][r] = mine[e];
