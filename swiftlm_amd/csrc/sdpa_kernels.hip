@@ -735,9 +735,9 @@ __global__ __launch_bounds__(kPartialThreads, 1) void sdpa_partial_kernel(SdpaAr
 
     // ---- epilogue: partial statistics and O rows (through LDS for coalesced stores) ----
     const float l_tot = l_run + __shfl_xor(l_run, 32);
-    if (row_valid && h == 0) {
-        A.part_m[row_id * A.S + split] = m_run;
-        A.part_l[row_id * A.S + split] = l_tot;
+    if (row_valid && h == 0) {      // written through like the partial rows: 4-byte fragments of lines shared with other splits
+        __hip_atomic_store(A.part_m + row_id * A.S + split, m_run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(A.part_l + row_id * A.S + split, l_tot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (wave_active) {
         const float inv_l = l_tot > 0.f ? 1.f / l_tot : 0.f;
