@@ -113,6 +113,19 @@ template <> __device__ __forceinline__ f16_t from_float<f16_t>(float f) { return
 template <typename T> __device__ __forceinline__ float requant(float f) { return to_float(from_float<T>(f)); }
 template <> __device__ __forceinline__ float requant<float>(float f) { return f; }
 
+// requant of four values at once; bf16 converts in pairs (one v_cvt_pk_bf16_f32 per two values, the same rounding)
+template <typename T> __device__ __forceinline__ float4 requant4(float4 v) {
+    return make_float4(requant<T>(v.x), requant<T>(v.y), requant<T>(v.z), requant<T>(v.w));
+}
+template <> __device__ __forceinline__ float4 requant4<bf16_t>(float4 v) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t lo = {v.x, v.y}, hi = {v.z, v.w};
+    const uint32_t a = __builtin_bit_cast(uint32_t, __builtin_convertvector(lo, bf16x2_t));
+    const uint32_t b = __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, bf16x2_t));
+    return make_float4(__uint_as_float(a << 16), __uint_as_float(a & 0xffff0000u), __uint_as_float(b << 16), __uint_as_float(b & 0xffff0000u));
+}
+
 // 4 consecutive elements -> float4 (pointer aligned to 4 elements)
 __device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
 __device__ __forceinline__ float4 load4(const bf16_t* p) {

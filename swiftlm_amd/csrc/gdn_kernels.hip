@@ -891,12 +891,29 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         const float alog = P.a_log[hv];
         const float dtb = P.dt_bias[hv];
         // ---- every load is out; now the arithmetic ----
+        // (pinned: left to itself the scheduler starts on the state tile, whose loads were first, before the last
+        //  window loads are issued, and those then leave a whole memory round trip later)
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
             const int i = tid + u * kThreads, r = i / (DK / 4), cc = (i % (DK / 4)) * 4;
             store_state4(r, cc, sv0[u]);
         }
         const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        // Without a carried window the rows in front of the sequence are zeros: set once here, under a uniform branch
+        // (selected tap by tap inside the conv it was a select per multiply on every call, carried window or not).
+        if (!cs) {
+#pragma unroll
+            for (int u = 0; u < NV; ++u) {
+                const int t = (tid + u * kThreads) / LPT, tl = t < tc ? t : tc - 1;
+#pragma unroll
+                for (int j = 0; j < KT; ++j)
+                    if (tl + j < keep) { kw[u][j] = zero4; qw[u][j] = zero4; }
+            }
+#pragma unroll
+            for (int j = 0; j < KT; ++j)
+                if (tvl + j < keep) vw[j] = 0.f;
+        }
         const bool first_tile = blockIdx.x == 0;
         const bool qk_owner = first_tile && (hv % (A.Hv / A.Hk)) == 0;
         auto conv4 = [&](const float4 (&w)[KT], const float4 (&tap)[4], int tl) -> float4 {
@@ -908,8 +925,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
 #pragma unroll
                 for (int j = 0; j < KT; ++j) {
                     const float wj[4] = {w[j].x, w[j].y, w[j].z, w[j].w};
-                    const float win = (tl + j < keep && !cs) ? 0.f : wj[m];
-                    acc = fmaf(win, tp[j], acc);
+                    acc = fmaf(wj[m], tp[j], acc);
                 }
                 o[m] = silu_f(acc);
             }
@@ -921,7 +937,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
             return gdn_norm_scale(butterfly_sum<LPT>(ss), DK, P.eps, sc);
         };
         auto round4 = [](float4 y, float sc) -> float4 {
-            return make_float4(requant<Elem>(y.x * sc), requant<Elem>(y.y * sc), requant<Elem>(y.z * sc), requant<Elem>(y.w * sc));
+            return requant4<Elem>(make_float4(y.x * sc, y.y * sc, y.z * sc, y.w * sc));
         };
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
@@ -938,9 +954,8 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
                     Elem* dst = reinterpret_cast<Elem*>(P.conv_out) + (size_t)b * keep * C;
 #pragma unroll
                     for (int j = 1; j < KT; ++j) {
-                        const bool z = (tl + j < keep && !cs);
-                        store4(dst + (size_t)(j - 1) * C + ck + c4, z ? zero4 : kw[u][j]);
-                        store4(dst + (size_t)(j - 1) * C + cq + c4, z ? zero4 : qw[u][j]);
+                        store4(dst + (size_t)(j - 1) * C + ck + c4, kw[u][j]);
+                        store4(dst + (size_t)(j - 1) * C + cq + c4, qw[u][j]);
                     }
                 }
             }
@@ -949,7 +964,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
             const float tp[4] = {vtap.x, vtap.y, vtap.z, vtap.w};
             float acc = 0.f;
 #pragma unroll
-            for (int j = 0; j < KT; ++j) acc = fmaf((tvl + j < keep && !cs) ? 0.f : vw[j], tp[j], acc);
+            for (int j = 0; j < KT; ++j) acc = fmaf(vw[j], tp[j], acc);
             const float vv = requant<Elem>(silu_f(acc));
             L.v[ts][tt] = ts < tc ? vv : 0.f;
             if (ts < tc) {
@@ -959,7 +974,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
                     Elem* dst = reinterpret_cast<Elem*>(P.conv_out) + (size_t)b * keep * C + cv + tt;
 #pragma unroll
                     for (int j = 1; j < KT; ++j)
-                        dst[(size_t)(j - 1) * C] = from_float<Elem>((tvl + j < keep && !cs) ? 0.f : vw[j]);
+                        dst[(size_t)(j - 1) * C] = from_float<Elem>(vw[j]);
                 }
             }
         }
