@@ -1255,6 +1255,11 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
                     cacc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, L.y[s][base + e], cacc[e], 0, 0, 0);
             }
             if (last_chunk) {
+                // (layer kernel with the gated norm inside: the wave's y rows and sums of squares must be acknowledged
+                //  before it counts itself in; waited for here, ahead of the state stores, the wait does not include
+                //  those)
+                if constexpr (FUSED)
+                    if (P.fin_gate) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
 #pragma unroll
@@ -1285,8 +1290,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         // workgroup that is not last is done.
         if constexpr (FUSED) {
             if (P.fin_gate) {
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                __syncthreads();
+                __builtin_amdgcn_s_barrier();       // every wave is past its wait for the y rows (the state stores may be in flight)
                 if (tid == 0) L.on[0] = __hip_atomic_fetch_add(P.arrivals + bh, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 __syncthreads();
                 if (L.on[0] != (int)gridDim.x - 1) return;
