@@ -377,6 +377,7 @@ def aux_gdn_layer(lib, cfg, n_layers=36, reps=30):
                    w=(0.5 * rn(C, Kc)).to(bf), a_log=0.5 * rn(Hv), dt_bias=rn(Hv), s0=0.1 * rn(B, Hv, Dv, Dk),
                    z=rn(B, T, Hv, Dv).to(bf), nw=(1 + 0.1 * rn(Dv)).to(bf)) for _ in range(n_layers)]
     sc = dict(q_scale=1.0 / Dk, k_scale=Dk ** -0.5)
+    arrivals = torch.zeros(B * Hv, dtype=torch.int32, device=dev)     # one array, zeroed once: every call leaves it zero
 
     def three(l):
         q, k, v, gg, beta, conv = K.gdn_prepare(l["x"], l["st"], l["w"], l["a"], l["b"], l["a_log"], l["dt_bias"], Hk, Hv, Dk, Dv, **sc)
@@ -385,7 +386,8 @@ def aux_gdn_layer(lib, cfg, n_layers=36, reps=30):
 
     def one(l, one_launch=True):
         r = K.gdn_layer(l["x"], l["st"], l["w"], l["a"], l["b"], l["a_log"], l["dt_bias"], l["s0"], Hk, Hv, Dk, Dv, **sc,
-                        gate=l["z"], norm_weight=l["nw"], norm_eps=1e-6, gate_kind="silu", one_launch=one_launch)
+                        gate=l["z"], norm_weight=l["nw"], norm_eps=1e-6, gate_kind="silu", one_launch=one_launch,
+                        arrivals=arrivals)
         return r["out"], r["state"], r["tape"], r["k"], r["g"], r["conv_state"]
 
     def two(l):              # the one call with the gated norm as a second launch

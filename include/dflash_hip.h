@@ -180,7 +180,15 @@ int dflash_gdn_finish(void* stream, const void* y, const void* gate, const void*
  *   arrivals  device int32 [B*Hv], all zero before the call; the call leaves it all zero, so one
  *             array zeroed once serves every later call that does not overlap with another one
  *             using the same array (calls on one stream never overlap).  NULL, or Dv > 256: the
- *             gated norm runs as a second launch, as dflash_gdn_finish.
+ *             gated norm runs as a second launch, as dflash_gdn_finish.  A counter that is not
+ *             zero when the launch begins (an array never cleared, or one a failed launch left
+ *             half counted) makes `out` of that head meaningless; a count the launch itself
+ *             cannot have produced sets DFLASH_STATUS_LAYER_ARRIVALS in the status word.
+ *   aliasing  until the last workgroup of a head has written it, each row of `out` carries
+ *             partial sums in its first Dv/16 floats.  The in-launch norm therefore needs `out`
+ *             4-byte aligned and disjoint from gate and out_norm_weight; when it is not (a caller
+ *             that norms in place, out == gate) the gated norm runs as the second launch, which
+ *             allows that aliasing, and the results are the same bits.  out may never overlap y_out.
  * Covers the verify block: float32 state, one decay per head and step, no step mask, K == 4,
  * T <= 16, Dk in {64, 128, 256}, Dv a multiple of 16.  Anything else returns
  * DFLASH_UNSUPPORTED and the caller issues the three calls.
@@ -419,38 +427,17 @@ int dflash_kv_append(void* stream, void* k_cache, void* v_cache, const void* k_n
  *                               was written and new_len_dev was left alone
  *   DFLASH_STATUS_CONV_STEPS    dflash_rebuild_conv_state found *steps_dev outside [0, T]: rows past the end of
  *                               the concatenation were left unwritten
+ *   DFLASH_STATUS_LAYER_ARRIVALS dflash_gdn_layer found an arrival counter at or above Dv/16, which no launch on a
+ *                               zeroed array produces: `arrivals` was not all zero before the call
+ * The pointer is read when a call is ENQUEUED and travels in the kernel's arguments: a captured HIP graph keeps the
+ * word that was registered at capture time and writes to it on every replay, so that word must outlive the graph
+ * (clearing or replacing the registration later does not reach launches already captured).
  * ---------------------------------------------------------------------- */
 #define DFLASH_STATUS_SDPA_LEN 1
 #define DFLASH_STATUS_APPEND_RANGE 2
 #define DFLASH_STATUS_CONV_STEPS 4
+#define DFLASH_STATUS_LAYER_ARRIVALS 8
 int dflash_set_status_word(int32_t* status_dev);
-
-/* ------------------------------------------------------------------------
- * Measurement hook (no counterpart in the reference, whose bench times whole
- * calls from the host: Sources/DFlashKernelBench/main.swift:33-57).  Arms the
- * calling thread so that the NEXT launch of the named kernel carries the two
- * events on its own dispatch (hipExtLaunchKernelGGL): their elapsed time is the
- * kernel's begin-to-end duration on the launch stream, as a profiler's kernel
- * trace reports it.  The arming is consumed by that launch.  Events are
- * hipEvent_t passed as void*, created and read by the caller.
- * ---------------------------------------------------------------------- */
-#define DFLASH_KERNEL_SDPA_PARTIAL 0
-#define DFLASH_KERNEL_SDPA_COMBINE 1
-#define DFLASH_KERNEL_GDN_FORWARD 2
-#define DFLASH_KERNEL_TAPE_REPLAY 3
-#define DFLASH_KERNEL_GREEDY_PARTIAL 4
-#define DFLASH_KERNEL_GDN_PREPARE 5
-#define DFLASH_KERNEL_EMPTY 6
-#define DFLASH_KERNEL_GDN_LAYER 7
-#define DFLASH_KERNEL_GDN_FINISH 8
-#define DFLASH_KERNEL_COUNT 9
-int dflash_profile_next_launch(int kernel_id, void* start_event, void* stop_event);
-
-/* Launches a kernel that does nothing, with the given grid, block size (a multiple of 64, at most
- * 1024) and dynamic LDS size (at most 160 KB): the cost of a launch of that shape before any work,
- * i.e. the floor under each kernel of a verify step.  No counterpart in the reference.  Kernel id
- * DFLASH_KERNEL_EMPTY for dflash_profile_next_launch. */
-int dflash_profile_empty_launch(void* stream, int grid_x, int grid_y, int grid_z, int threads, int lds_bytes);
 
 #ifdef __cplusplus
 }

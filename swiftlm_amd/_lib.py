@@ -1,5 +1,5 @@
 """ctypes binding of libdflash_hip.so, the C ABI declared in include/dflash_hip.h
-and include/dflash_cache.h.
+and include/dflash_cache.h (plus the measurement hooks of include/dflash_profile.h).
 
 There is no CPU or PyTorch fallback anywhere in this package: if the library is
 not built, or the device is not a gfx950, loading fails with an error.
@@ -17,7 +17,7 @@ OK, UNSUPPORTED, INVALID = 0, 1, 2
 F32, BF16, F16, U8 = 0, 1, 2, 3
 CACHE_TAPE, CACHE_SNAPSHOT, CACHE_MAMBA, CACHE_KV = 0, 1, 2, 3
 MAX_BATCHED_LAYERS = 64
-STATUS_SDPA_LEN, STATUS_APPEND_RANGE, STATUS_CONV_STEPS = 1, 2, 4
+STATUS_SDPA_LEN, STATUS_APPEND_RANGE, STATUS_CONV_STEPS, STATUS_LAYER_ARRIVALS = 1, 2, 4, 8
 KERNEL_SDPA_PARTIAL, KERNEL_SDPA_COMBINE, KERNEL_GDN_FORWARD, KERNEL_TAPE_REPLAY = 0, 1, 2, 3
 KERNEL_GREEDY_PARTIAL, KERNEL_GDN_PREPARE, KERNEL_EMPTY, KERNEL_GDN_LAYER, KERNEL_GDN_FINISH = 4, 5, 6, 7, 8
 

@@ -10,6 +10,7 @@
 #include <stdio.h>
 
 #include "../../include/dflash_hip.h"
+#include "../../include/dflash_profile.h"
 
 namespace dflash {
 

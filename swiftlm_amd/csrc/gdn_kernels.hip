@@ -426,6 +426,7 @@ struct GdnPrep {
     void* fin_out;            // [B,T,Hv,Dv]; until the last workgroup writes a row, its first Dv/16 floats hold
                               // the row tiles' sums of squares
     int32_t* arrivals;        // [B*Hv]
+    int32_t* status;          // device status word (dflash_set_status_word), or null
     float fin_eps;
     int fin_silu;
 };
@@ -705,7 +706,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
                      "s"(P.dt_bias), "s"(P.q_out), "s"(P.k_out), "s"(P.v_out), "s"(P.g_out), "s"(P.beta_out), "s"(P.conv_out),
                      "s"(P.q_scale), "s"(P.k_scale), "s"(P.eps), "s"(P.C));
     if constexpr (FUSED)
-        asm volatile("" ::"s"(P.fin_gate), "s"(P.fin_weight), "s"(P.fin_out), "s"(P.arrivals), "s"(P.fin_eps), "s"(P.fin_silu));
+        asm volatile("" ::"s"(P.fin_gate), "s"(P.fin_weight), "s"(P.fin_out), "s"(P.arrivals), "s"(P.status), "s"(P.fin_eps), "s"(P.fin_silu));
     if constexpr (!FUSED)
         asm volatile("" ::"s"(A.q), "s"(A.k), "s"(A.v), "s"(A.g), "s"(A.beta), "s"(A.mask), "s"(A.state_in), "s"(A.state_out),
                      "s"(A.y), "s"(A.tape), "s"(A.in_dtype), "s"(A.mask_dtype), "s"(A.T), "s"(A.Hk), "s"(A.Hv), "s"(A.Dv),
@@ -1284,17 +1285,34 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         }
 
         // ---- the layer's post-op, by the head's last workgroup ----
-        // Every workgroup of the head has written its y rows and sums of squares through to agent scope; once those
-        // stores are acknowledged it counts itself in, and the one that finds all others already counted re-reads
-        // the head's y (at agent scope), finishes the sums and writes `out`.  Nothing waits for anything: a
-        // workgroup that is not last is done.
+        // The hand-over between the workgroups of a head, in the order that makes it correct:
+        //   1. store    every producer writes its y rows and sums of squares with agent-scope stores, which go through
+        //               its XCD's L2 to the memory side that all XCDs share;
+        //   2. ack      it waits until the memory side has acknowledged them (vmcnt(0), above, then the barrier below:
+        //               every wave of the workgroup is past its own wait);
+        //   3. count    only then does it add itself to the head's counter (an agent-scope read-modify-write, performed
+        //               at that same shared level, hence ordered behind the acknowledged stores);
+        //   4. observe  the workgroup whose own increment returns tiles - 1 has observed the increments of all others,
+        //               each of which was issued behind that workgroup's acknowledged stores;
+        //   5. acquire  it invalidates what its own caches may hold of those lines (an agent-scope acquire fence: an
+        //               invalidate, not a write-back -- paid by one workgroup per head);
+        //   6. load     and re-reads the head's y and the parked sums (agent-scope loads), finishes the sums, writes `out`.
+        // Steps 1-3 are a release of exactly the lines that are handed over (a release FENCE would also write back the
+        // 2 MB of new state every workgroup has dirtied: 30 us per launch); 4-6 are the matching acquire.  Nothing
+        // waits for anything: a workgroup that is not last is done.
         if constexpr (FUSED) {
             if (P.fin_gate) {
                 __builtin_amdgcn_s_barrier();       // every wave is past its wait for the y rows (the state stores may be in flight)
                 if (tid == 0) L.on[0] = __hip_atomic_fetch_add(P.arrivals + bh, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 __syncthreads();
-                if (L.on[0] != (int)gridDim.x - 1) return;
+                const int arrived = L.on[0];
+                // A count this launch cannot have produced: the array was not zero when the launch began (never
+                // cleared, or left behind by a launch that did not finish).  `out` of this head is then not to be
+                // trusted; say so where the caller can see it.
+                if (arrived >= (int)gridDim.x && P.status && tid == 0) atomicOr(P.status, DFLASH_STATUS_LAYER_ARRIVALS);
+                if (arrived != (int)gridDim.x - 1) return;
                 if (tid == 0) __hip_atomic_store(P.arrivals + bh, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // as the next launch expects it
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
                 if (A.in_dtype == DFLASH_BF16) finish_head(bf16_t{}, tc);
                 else if (A.in_dtype == DFLASH_F16) finish_head(f16_t{}, tc);
                 else finish_head(float{}, tc);
@@ -1514,11 +1532,23 @@ extern "C" int dflash_gdn_layer(void* stream, const void* mixed_qkv, const void*
     P.C = 2 * Hk * Dk + Hv * Dv;
     // With a counter array the post-op runs inside the same launch; without one (or with a head dim the kernel's
     // post-op is not unrolled for) it is a second launch.
-    const bool finish_inside = gate && arrivals && Dv <= kLayerFinishMaxDv;
+    // While the launch runs, the first Dv/16 floats of every row of `out` hold the row tiles' sums of squares, so the
+    // in-launch norm needs `out` to be 4-byte aligned and disjoint from everything the last workgroup still reads
+    // (gate, the norm weight); a caller that norms in place (out == gate) gets the second launch, which allows it.
+    const size_t esz = in_dtype == DFLASH_F32 ? 4 : 2;
+    const size_t out_bytes = (size_t)B * T * Hv * Dv * esz;
+    auto overlaps = [&](const void* p, size_t bytes) {
+        const uintptr_t a = (uintptr_t)out, b = (uintptr_t)p;
+        return p && a < b + bytes && b < a + out_bytes;
+    };
+    DFLASH_REQUIRE(!gate || !overlaps(y_out, out_bytes), "gdn_layer: out overlaps y_out");
+    const bool out_private = gate && (uintptr_t)out % 4 == 0 && !overlaps(gate, out_bytes) && !overlaps(out_norm_weight, (size_t)Dv * esz);
+    const bool finish_inside = gate && arrivals && Dv <= kLayerFinishMaxDv && out_private;
     P.fin_gate = finish_inside ? gate : nullptr;
     P.fin_weight = finish_inside ? out_norm_weight : nullptr;
     P.fin_out = finish_inside ? out : nullptr;
     P.arrivals = finish_inside ? arrivals : nullptr;
+    P.status = status_word();
     P.fin_eps = out_norm_eps;
     P.fin_silu = gate_kind;
     hipStream_t st = (hipStream_t)stream;

@@ -198,7 +198,8 @@ class DFlashKernels:
                   state: torch.Tensor, Hk: int, Hv: int, Dk: int, Dv: int, q_scale: float, k_scale: float,
                   eps: float = 1e-6, gate: Optional[torch.Tensor] = None, norm_weight: Optional[torch.Tensor] = None,
                   norm_eps: float = 1e-6, gate_kind: str = "sigmoid", want_intermediates: bool = False,
-                  arrivals: Optional[torch.Tensor] = None, one_launch: bool = True):
+                  arrivals: Optional[torch.Tensor] = None, one_launch: bool = True,
+                  out: Optional[torch.Tensor] = None):
         """The body of a GatedDelta layer between its projections (KimiLinearDFlash.swift:351-378) in one
         call: ``gdn_prepare`` -> ``gated_delta_kernel_with_tape`` -> ``gdn_finish`` with the pre-ops done
         inside the forward kernel.  Returns a dict: ``out`` (None without ``gate``), ``y``, ``state``,
@@ -209,7 +210,8 @@ class DFlashKernels:
         With a ``gate`` the gated norm runs inside the same launch, done by the last workgroup of each head;
         the heads' arrival counters are ``arrivals`` (int32 [B*Hv], zero before and after every call) or, when
         it is None, an array this module keeps per device, stream and size.  ``one_launch=False`` runs the gated
-        norm as a second launch instead."""
+        norm as a second launch instead.  ``out`` (optional, [B,T,Hv,Dv] in the input type) receives the gated norm
+        instead of a fresh tensor; it may be ``gate`` itself (the library then takes the second launch)."""
         _dev(mixed_qkv, conv_state, conv_weight, a_logits, b_logits, a_log, dt_bias, state, gate, norm_weight)
         B, T, C = mixed_qkv.shape
         if C != 2 * Hk * Dk + Hv * Dv:
@@ -238,18 +240,28 @@ class DFlashKernels:
         q = torch.empty_like(k) if want_intermediates else None
         v = torch.empty_like(y) if want_intermediates else None
         beta = torch.empty_like(g) if want_intermediates else None
-        out = zg = nw = None
+        zg = nw = None
+        if gate is None:
+            out = None
         if gate is not None:
             if norm_weight is None or gate.shape != y.shape or norm_weight.shape != (Dv,):
                 raise DFlashError("gdn_layer: gate must be [B,T,Hv,Dv] and come with norm_weight [Dv]")
             zg, nw = gate.to(dt).contiguous(), norm_weight.to(dt).contiguous()
-            out = torch.empty_like(y)
+            if out is None:
+                out = torch.empty_like(y)
+            elif out.shape != y.shape or out.dtype != dt or not out.is_contiguous() or not out.is_cuda:
+                raise DFlashError("gdn_layer: out must be a contiguous device tensor [B,T,Hv,Dv] of the input type")
             if not one_launch:
                 arrivals = None
             elif arrivals is None:
                 key = (dv.index, torch.cuda.current_stream().cuda_stream, B * Hv)
                 arrivals = _ARRIVALS.get(key)
                 if arrivals is None:
+                    if torch.cuda.is_current_stream_capturing():
+                        # zeros created here would only be RECORDED (and live in the graph's private pool): an eager call
+                        # on this stream before the first replay would count into uninitialised memory
+                        raise DFlashError("gdn_layer: first use on this stream happens inside a graph capture; pass "
+                                          "`arrivals` (int32 zeros [B*Hv]) or call gdn_layer once on this stream beforehand")
                     arrivals = _ARRIVALS[key] = torch.zeros(B * Hv, dtype=torch.int32, device=dv)
             elif arrivals.dtype != torch.int32 or arrivals.numel() < B * Hv or not arrivals.is_contiguous():
                 raise DFlashError("gdn_layer: arrivals must be a contiguous int32 tensor of at least B*Hv elements")

@@ -16,7 +16,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def _declared_symbols():
     names = set()
-    for h in ("dflash_hip.h", "dflash_cache.h"):
+    for h in ("dflash_hip.h", "dflash_cache.h", "dflash_profile.h"):
         text = open(os.path.join(ROOT, "include", h)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         names |= set(re.findall(r"\b(dflash_[a-z0-9_]+)\s*\(", text))

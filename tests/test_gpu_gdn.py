@@ -404,3 +404,178 @@ def test_gdn_layer_reports_unsupported_outside_the_verify_block(gpu_lib):
         args = [dev(d[n], "bf16") for n in ("x", "state", "w", "a", "b")] + [dev(d["a_log"]), dev(d["dt_bias"])]
         with pytest.raises(DFlashUnsupported):
             K.gdn_layer(*args, torch.zeros(B, Hv, Dv, Dk, device="cuda"), Hk, Hv, Dk, Dv, q_scale=1.0, k_scale=1.0)
+
+
+def _layer_case(seed, B, T, Hk, Hv, Dk, Dv, in_dt="bf16"):
+    """Device inputs of one layer call plus the three-call result they must reproduce."""
+    from swiftlm_amd import DFlashKernels as K
+
+    d = _prep_inputs(seed, B, T, Hk, Hv, Dk, Dv, 4, False)
+    rd = {"f32": lambda a: a, "bf16": O.round_to_bf16, "f16": lambda a: a.astype(np.float16).astype(np.float32)}[in_dt]
+    x, st, w, a, bl = (dev(rd(d[n]), in_dt) for n in ("x", "state", "w", "a", "b"))
+    rng = np.random.default_rng(seed + 1)
+    s0 = dev(0.1 * rng.standard_normal((B, Hv, Dv, Dk)).astype(np.float32))
+    z = dev(rd((rng.standard_normal((B, T, Hv, Dv)) * 2).astype(np.float32)), in_dt)
+    nw = dev(rd((1 + 0.1 * rng.standard_normal(Dv)).astype(np.float32)), in_dt)
+    sc = dict(q_scale=1.0 / Dk, k_scale=Dk ** -0.5)
+    args = (x, st, w, a, bl, dev(d["a_log"]), dev(d["dt_bias"]), s0, Hk, Hv, Dk, Dv)
+    kw = dict(**sc, gate=z, norm_weight=nw, norm_eps=1e-6, gate_kind="silu")
+    q, k, v, g, beta, conv1 = K.gdn_prepare(x, st, w, a, bl, dev(d["a_log"]), dev(d["dt_bias"]), Hk, Hv, Dk, Dv, **sc)
+    y, s1, tape = K.gated_delta_kernel_with_tape(q, k, v, g, beta, s0)
+    out = K.gdn_finish(y, z, nw, 1e-6, "silu")
+    want = dict(out=out, y=y, state=s1, tape=tape, k=k, g=g, conv_state=conv1)
+    return args, kw, want
+
+
+def _assert_layer_equals(r, want, what=""):
+    for name, w in want.items():
+        assert torch.equal(r[name], w), f"{name} {what}"
+
+
+@pytest.mark.parametrize("cfg", [(1, 16, 2, 4, 128, 256), (1, 16, 2, 2, 128, 272), (1, 8, 1, 2, 64, 512), (2, 16, 16, 32, 128, 128)],
+                         ids=["dv256_widest_in_launch_norm", "dv272_second_launch", "dv512_second_launch", "64_heads"])
+def test_gdn_layer_widest_norm_fallback_and_many_heads(gpu_lib, cfg):
+    """The in-launch gated norm at the widest head it is unrolled for (Dv = 256: 16 row tiles per head), the
+    automatic second launch beyond that, and 64 heads counting into ONE arrivals array over six back-to-back calls."""
+    from swiftlm_amd import DFlashKernels as K
+
+    B, T, Hk, Hv, Dk, Dv = cfg
+    args, kw, want = _layer_case(77 + Dv, B, T, Hk, Hv, Dk, Dv)
+    arrivals = torch.zeros(B * Hv, dtype=torch.int32, device="cuda")
+    runs = [K.gdn_layer(*args, **kw, arrivals=arrivals) for _ in range(6)]
+    torch.cuda.synchronize()
+    assert not arrivals.any()
+    for i, r in enumerate(runs):
+        _assert_layer_equals(r, want, f"(call {i})")
+    pre = K.gdn_prepare(*args[:7], Hk, Hv, Dk, Dv, q_scale=1.0 / Dk, k_scale=Dk ** -0.5)
+    yw, sw, tw = O.gated_delta_ops_with_tape(*(host(t) for t in pre[:5]), host(args[7]), dtype=np.float64)
+    np.testing.assert_allclose(host(runs[0]["state"]), sw, **STATE_TOL)     # the equality is not two wrong answers agreeing
+
+
+def test_gdn_layer_out_aliasing_gate_or_misaligned_takes_the_second_launch(gpu_lib):
+    """While the launch runs, `out` carries partial sums; a caller that norms in place (out is gate) or hands a
+    2-byte-aligned `out` must still get the three-call bits (the library then runs the norm as a second launch)."""
+    from swiftlm_amd import DFlashKernels as K, DFlashError
+
+    B, T, Hk, Hv, Dk, Dv = 1, 16, 4, 8, 128, 128
+    args, kw, want = _layer_case(5, B, T, Hk, Hv, Dk, Dv)
+    arrivals = torch.zeros(B * Hv, dtype=torch.int32, device="cuda")
+    gate_copy = kw["gate"].clone()
+    kw_alias = dict(kw, gate=gate_copy)
+    r = K.gdn_layer(*args, **kw_alias, arrivals=arrivals, out=gate_copy)          # in place
+    torch.cuda.synchronize()
+    assert r["out"].data_ptr() == gate_copy.data_ptr()
+    _assert_layer_equals(r, want, "(out is gate)")
+    odd = torch.empty(B * T * Hv * Dv + 1, dtype=torch.bfloat16, device="cuda")[1:].view(B, T, Hv, Dv)
+    assert odd.data_ptr() % 4 == 2
+    r = K.gdn_layer(*args, **kw, arrivals=arrivals, out=odd)
+    torch.cuda.synchronize()
+    _assert_layer_equals(r, want, "(out 2-byte aligned)")
+    assert not arrivals.any()
+    # out overlapping y_out cannot be served by either form; the mirror allocates y itself, so go through the C ABI
+    from swiftlm_amd import _lib
+    from swiftlm_amd.dflash_kernels import _ptr, _stream
+    x, st, w, a, bl, al, db, s0 = args[:8]
+    C = x.shape[-1]
+    y = torch.empty(B, T, Hv, Dv, dtype=torch.bfloat16, device="cuda")
+    rc = _lib.load().dflash_gdn_layer(
+        _stream(), _ptr(x), _ptr(st), _ptr(w), _ptr(a), _ptr(bl), _ptr(al), _ptr(db), _lib.BF16, 1.0 / Dk, Dk ** -0.5, 1e-6,
+        _ptr(s0), _ptr(torch.empty_like(s0)), None, None, _ptr(torch.empty(B, T, Hv, Dv, device="cuda")),
+        _ptr(torch.empty(B, 3, C, dtype=torch.bfloat16, device="cuda")), _ptr(y), _ptr(kw["gate"]), _ptr(kw["norm_weight"]), 1e-6, 1,
+        _ptr(y.view(-1)[8:]), _ptr(arrivals), None, None, None, B, T, Hk, Hv, Dk, Dv, 4)
+    assert rc == _lib.INVALID and "overlaps y_out" in _lib.last_error()
+
+
+def test_gdn_layer_flags_an_arrivals_array_that_was_not_zero(gpu_lib):
+    from swiftlm_amd import DFlashKernels as K, _lib
+    from swiftlm_amd.dflash_kernels import _ptr
+
+    B, T, Hk, Hv, Dk, Dv = 1, 16, 2, 4, 128, 64
+    args, kw, want = _layer_case(6, B, T, Hk, Hv, Dk, Dv)
+    lib = _lib.load()
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    assert lib.dflash_set_status_word(_ptr(status)) == 0
+    try:
+        arrivals = torch.zeros(B * Hv, dtype=torch.int32, device="cuda")
+        _assert_layer_equals(K.gdn_layer(*args, **kw, arrivals=arrivals), want)
+        torch.cuda.synchronize()
+        assert int(status) == 0                                  # in contract: no flag
+        garbage = torch.full((B * Hv,), 1000, dtype=torch.int32, device="cuda")
+        r = K.gdn_layer(*args, **kw, arrivals=garbage)
+        torch.cuda.synchronize()
+        assert int(status) == _lib.STATUS_LAYER_ARRIVALS
+        for name in ("y", "state", "tape", "k", "g", "conv_state"):      # everything but the gated norm is unaffected
+            assert torch.equal(r[name], want[name]), name
+    finally:
+        lib.dflash_set_status_word(None)
+
+
+def test_gdn_layer_inside_a_capture_needs_its_counters_from_outside(gpu_lib):
+    """On a stream the module has not served yet, a capture cannot create the counters (their zero-fill would only
+    be recorded): the mirror refuses; with a caller-provided array the captured call replays to the eager bits."""
+    from swiftlm_amd import DFlashKernels as K, DFlashError
+
+    B, T, Hk, Hv, Dk, Dv = 1, 16, 2, 4, 128, 64
+    args, kw, want = _layer_case(8, B, T, Hk, Hv, Dk, Dv)
+    fresh = torch.cuda.Stream()
+    fresh.wait_stream(torch.cuda.current_stream())
+    arrivals = torch.zeros(B * Hv, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=fresh):
+        with pytest.raises(DFlashError, match="inside a graph capture"):
+            K.gdn_layer(*args, **kw)
+        r = K.gdn_layer(*args, **kw, arrivals=arrivals)
+    for i in range(3):
+        for t in r.values():
+            if t is not None:
+                t.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        _assert_layer_equals(r, want, f"(replay {i})")
+        assert not arrivals.any()
+
+
+def test_gdn_layer_hand_over_holds_over_many_graph_launches(gpu_lib):
+    """The Qwen3-Next block through the one-launch layer 320 times inside captured graphs (8 graphs x 40 layer
+    launches, each followed by other kernels: a fill of the previous result and a tape replay that dirties the L2s),
+    compared bit for bit with the three-call result; stops at the first mismatch."""
+    from swiftlm_amd import DFlashKernels as K
+
+    B, T, Hk, Hv, Dk, Dv = 1, 16, 16, 32, 128, 128
+    cases = [_layer_case(900 + i, B, T, Hk, Hv, Dk, Dv) for i in range(4)]
+    arrivals = torch.zeros(B * Hv, dtype=torch.int32, device="cuda")
+    for args, kw, _ in cases:                                    # code objects loaded, attributes set: nothing to set up inside a capture
+        K.gdn_layer(*args, **kw, arrivals=arrivals)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    side.wait_stream(torch.cuda.current_stream())
+    per_graph = 40
+    g = torch.cuda.CUDAGraph()
+    scratch_state = torch.empty(B, Hv, Dv, Dk, device="cuda")
+    with torch.cuda.graph(g, stream=side):
+        results = []
+        for i in range(per_graph):
+            args, kw, want = cases[i % len(cases)]
+            r = K.gdn_layer(*args, **kw, arrivals=arrivals)
+            results.append((r, want))
+            # other work between the layer launches: a replay over the fresh tape (reads what the layer wrote,
+            # writes 2 MB elsewhere) and a fill
+            K.tape_replay_batched([r["tape"]], [r["k"]], [r["g"]], [args[7]], [scratch_state], 3)
+            scratch_state.mul_(0.5)
+    torch.cuda.current_stream().wait_stream(side)
+    launches = 0
+    for rep in range(8):
+        for r, _ in results:
+            r["out"].fill_(float("nan"))
+        g.replay()
+        torch.cuda.synchronize()
+        for i, (r, want) in enumerate(results):
+            launches += 1
+            for name, w in want.items():
+                if not torch.equal(r[name], w):
+                    bad = (r[name].float() - w.float()).abs()
+                    pytest.fail(f"replay {rep}, layer launch {i}: {name} differs from the three calls "
+                                f"({int((bad > 0).sum())} elements, max abs {float(bad.max()):.3e})")
+        assert not arrivals.any()
+    assert launches == 320

@@ -25,6 +25,23 @@ def host(t):
     return t.detach().float().cpu().numpy()
 
 
+def torch_reference(q, k, v, scale, kv_len):
+    """float32 restatement on the GPU over the first kv_len[b] keys of each sequence."""
+    B, Hq, M, D = q.shape
+    Hk = k.shape[1]
+    outs, lses = [], []
+    for b in range(B):
+        n = int(kv_len[b])
+        kk = k[b, :, :n].float().repeat_interleave(Hq // Hk, dim=0)
+        vv = v[b, :, :n].float().repeat_interleave(Hq // Hk, dim=0)
+        s = torch.einsum("hmd,hnd->hmn", q[b].float() * scale, kk)
+        vis = torch.arange(n, device=q.device)[None, :] <= (n - M + torch.arange(M, device=q.device))[:, None]
+        s = s.masked_fill(~vis, float("-inf"))
+        lses.append(torch.logsumexp(s, dim=-1))
+        outs.append(torch.einsum("hmn,hnd->hmd", torch.softmax(s, dim=-1), vv))
+    return torch.stack(outs), torch.stack(lses)
+
+
 def paged_case(seed, B, Hq, Hk, lengths, D, page_size, dtype=torch.bfloat16, spare_pages=3, head_pad=0, page_pad=0):
     """Dense K/V per sequence plus a pool that holds them under a shuffled page table.
     lengths: keys per sequence, block included.  head_pad / page_pad add unused elements to the
@@ -287,3 +304,51 @@ def test_paged_random_shapes(gpu_lib, seed):
             ref, ref_lse = O.sdpa_block_causal(host(q[b:b + 1]), kd, vd, scale)
             np.testing.assert_allclose(host(got[b:b + 1]), ref, err_msg=case, **OUT_TOL)
             np.testing.assert_allclose(host(got_lse[b:b + 1]), ref_lse, err_msg=case, **LSE_TOL)
+
+
+@pytest.mark.parametrize("variant", ["plain", "masked", "append", "paged", "paged_append"])
+@pytest.mark.parametrize("D", [128, 256])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_device_side_length_shorter_than_bound_in_every_instantiation(gpu_lib, variant, D, dtype):
+    """Every instantiation of the partial kernel (two element types x two head dims x plain / masked / paged, with
+    and without the fused append) reads the per-sequence key count from device memory through the scalar cache and
+    waits for it by hand.  Each is run with ragged counts well below the host-side bound N -- a count taken too early
+    would attend N keys (or garbage) -- and checked against the float32 restatement on exactly the live keys."""
+    from swiftlm_amd import DFlashKernels as K
+
+    B, Hq, Hk, P = 3, 8, 2, 64
+    lens = [16 + 37, 16 + 700, 16 + 1501]                      # keys per sequence, block included
+    N = 2000                                                   # the host-side bound (a cache capacity), never reached
+    q, k, v, k_pool, v_pool, table = paged_case(D + len(variant), B, Hq, Hk, [N] * B, D, P, dtype)
+    scale = 1.0 / math.sqrt(D)
+    kv_len = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    cache_len = kv_len - 16
+    g = torch.Generator(device="cuda").manual_seed(4)
+    k_new = torch.randn(B, Hk, 16, D, generator=g, device="cuda").to(dtype)
+    v_new = torch.randn(B, Hk, 16, D, generator=g, device="cuda").to(dtype)
+    if "append" in variant:                                    # what the attention must see: the block's rows at cache_len
+        for b in range(B):
+            k[b, :, lens[b] - 16:lens[b]] = k_new[b]
+            v[b, :, lens[b] - 16:lens[b]] = v_new[b]
+    ow, lw = torch_reference(q, k, v, scale, kv_len=lens)
+    if variant == "plain":
+        out, lse = K.batched_sdpa_2pass(q, k, v, scale, return_lse=True, kv_len=kv_len)
+    elif variant == "masked":
+        zero = torch.zeros(B, Hq, 16, N, dtype=dtype, device="cuda")
+        out, lse = K.batched_sdpa_2pass(q, k, v, scale, zero, return_lse=True, kv_len=kv_len)
+    elif variant == "append":
+        kc, vc = k.clone(), v.clone()
+        for b in range(B):                                     # the cache does not hold the block yet
+            kc[b, :, lens[b] - 16:lens[b]] = 0
+            vc[b, :, lens[b] - 16:lens[b]] = 0
+        out, lse = K.batched_sdpa_2pass_append(q, kc, vc, k_new, v_new, scale, N, return_lse=True, cache_len=cache_len)
+        for b in range(B):
+            assert torch.equal(kc[b, :, lens[b] - 16:lens[b]], k_new[b]) and torch.equal(vc[b, :, lens[b] - 16:lens[b]], v_new[b])
+    elif variant == "paged":
+        out, lse = K.batched_sdpa_2pass_paged(q, k_pool, v_pool, table, scale, N, lengths=kv_len, return_lse=True)
+    else:
+        out, lse = K.batched_sdpa_2pass_paged(q, k_pool, v_pool, table, scale, N, k_new=k_new, v_new=v_new,
+                                              lengths=cache_len, return_lse=True)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(host(out), host(ow), **OUT_TOL)
+    np.testing.assert_allclose(host(lse), host(lw), **LSE_TOL)

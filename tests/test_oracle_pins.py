@@ -166,6 +166,36 @@ def test_gated_delta_matches_matrix_form(vec):
     np.testing.assert_allclose(tape, tw, rtol=1e-11, atol=1e-13)
 
 
+@pytest.mark.parametrize("vec", [False, True])
+def test_signed_and_degenerate_gates_match_matrix_and_closed_forms(vec):
+    """The reference micro-benchmark draws EVERYTHING from uniform(-0.1, 0.1), gates and betas included
+    (Sources/DFlashKernelBench/main.swift:28-30), so the oracle must hold for negative decays and betas and for
+    the degenerate values 0 and 1: checked against the matrix form of the delta rule and, for the replay, the
+    closed form (neither takes a logarithm, a quotient or a root of a gate)."""
+    rng = np.random.default_rng(21)
+    B, T, Hk, Hv, Dk, Dv = 2, 7, 2, 4, 8, 5
+    u = lambda *s: rng.uniform(-0.1, 0.1, s).astype(np.float32)
+    gshape = (B, T, Hv, Dk) if vec else (B, T, Hv)
+    q, k, v, g, beta, S0 = u(B, T, Hk, Dk), u(B, T, Hk, Dk), u(B, T, Hv, Dv), u(*gshape), u(B, T, Hv), u(B, Hv, Dv, Dk)
+    g[:, 1], g[:, 3], g[:, 5] = 0.0, 1.0, -0.5
+    beta[:, 2], beta[:, 4] = 0.0, 1.0
+    y, S, tape = O.gated_delta_ops_with_tape(q, k, v, g, beta, S0, dtype=F64)
+    yw, Sw, tw = _matrix_form(q, k, v, g, beta, S0)
+    np.testing.assert_allclose(y, yw, rtol=1e-11, atol=1e-15)
+    np.testing.assert_allclose(S, Sw, rtol=1e-11, atol=1e-15)
+    np.testing.assert_allclose(tape, tw, rtol=1e-11, atol=1e-15)
+    # replay of that tape: closed form with suffix products of the signed gates
+    got = O.tape_replay_ops(tape, k, g, S0, dtype=F64)
+    gg = g.astype(F64) if vec else np.broadcast_to(g.astype(F64)[..., None], (B, T, Hv, Dk))
+    c = np.ones_like(gg)
+    for t in range(T - 2, -1, -1):
+        c[:, t] = c[:, t + 1] * gg[:, t + 1]
+    k_rep = np.repeat(k.astype(F64), Hv // Hk, axis=2)
+    want = gg.prod(axis=1)[:, :, None, :] * S0.astype(F64) + np.einsum("bthk,bthv,bthk->bhvk", c, tape, k_rep)
+    np.testing.assert_allclose(got, want, rtol=1e-11, atol=1e-15)
+    np.testing.assert_allclose(got, S, rtol=1e-11, atol=1e-15)        # and it lands on the forward's state
+
+
 def test_gated_delta_matches_kimi_restatement():
     # Second in-tree statement of the recurrence, vector gate, Hk == Hv
     # (Sources/SwiftLM/KimiLinearDFlash.swift:395-403), written with einsum.
