@@ -455,7 +455,80 @@ def side_config(lib, name, reps=40):
         ev.destroy()
         return {"median_us": round(float(np.median(d)), 2), "min_us": round(float(d.min()), 2), "launches": len(d)}
 
-    if name == "config1":
+    if name == "refbench":
+        # The shapes and the input distribution of the reference's own micro-benchmark
+        # (Sources/DFlashKernelBench/main.swift): everything uniform(-0.1, 0.1) in bf16 (:28-30), recurrences at
+        # B=1 T=16 Hk=8 Hv=16 Dk=Dv=128 with a bf16 state and a bf16 tape (:107-117, :150-157), masked and unmasked
+        # (mask = uniform >= 0.5, :117), attention at Hq=32 Hk=8 D=128 over nKV keys, block included (:201-213).  The
+        # two figures the reference records for this path -- 382 us replay / 816 us forward, ops fallback, masked
+        # scalar gate, "M-series" (DFlashKernels.swift:400-401, :447-448) -- are at the recurrence shape; the C
+        # restatement of that ops path is timed beside the kernels on this box's host cores.
+        from oracle import c_oracle
+        B, T, Hk, Hv, Dk, Dv = 1, 16, 8, 16, 128, 128
+        u = lambda *shape: (torch.rand(*shape, generator=g, device=dev) * 0.2 - 0.1).to(bf)
+        nset = 24
+        sets = [dict(q=u(B, T, Hk, Dk), k=u(B, T, Hk, Dk), v=u(B, T, Hv, Dv), g=u(B, T, Hv), gv=u(B, T, Hv, Dk), beta=u(B, T, Hv),
+                     tape=u(B, T, Hv, Dv), state=u(B, Hv, Dv, Dk),
+                     mask=(torch.rand(B, T, generator=g, device=dev) >= 0.5).to(bf)) for _ in range(nset)]
+        state_b = lambda sb: 2 * B * Hv * Dv * Dk * sb
+        replay_bytes = lambda sb, tb: state_b(sb) + T * (B * Hv * Dv * tb + B * Hk * Dk * 2 + B * Hv * 2)
+        fwd_bytes = lambda sb: state_b(sb) + (2 * T * Hk * Dk + T * Hv * Dv + 2 * T * Hv) * 2 + T * Hv * Dv * 2 + T * Hv * Dv * 4
+        rec = {}
+        for label, cast, sb in (("bf16_state_as_the_reference_bench_passes_it", lambda t: t, 2), ("fp32_state", lambda t: t.float(), 4)):
+            for mname, mk in (("", lambda d: None), ("_masked", lambda d: d["mask"])):
+                calls = [(lambda d=d: K.tape_replay_kernel(cast(d["tape"]), d["k"], d["g"], cast(d["state"]), mk(d))) for d in sets] * 2
+                r = timed(_lib.KERNEL_TAPE_REPLAY, calls)
+                r["algorithmic_bytes"] = replay_bytes(sb, sb)
+                r["gbs"] = round(r["algorithmic_bytes"] / r["median_us"] / 1e3, 1)
+                rec["tape_replay_scalar_g%s_%s" % (mname, label)] = r
+                calls = [(lambda d=d: K.gated_delta_kernel_with_tape(d["q"], d["k"], d["v"], d["g"], d["beta"], cast(d["state"]), mk(d)))
+                         for d in sets] * 2
+                r = timed(_lib.KERNEL_GDN_FORWARD, calls)
+                r["algorithmic_bytes"] = fwd_bytes(sb)
+                r["gbs"] = round(r["algorithmic_bytes"] / r["median_us"] / 1e3, 1)
+                rec["gated_delta_tape_scalar_g%s_%s" % (mname, label)] = r
+        calls = [(lambda d=d: K.tape_replay_kernel(d["tape"], d["k"], d["gv"], d["state"])) for d in sets] * 2
+        rec["tape_replay_vec_g_bf16_state"] = timed(_lib.KERNEL_TAPE_REPLAY, calls)
+        calls = [(lambda d=d: K.gated_delta_kernel_with_tape(d["q"], d["k"], d["v"], d["gv"], d["beta"], d["state"])) for d in sets] * 2
+        rec["gated_delta_tape_vec_g_bf16_state"] = timed(_lib.KERNEL_GDN_FORWARD, calls)
+        out["recurrences"] = rec
+        out["recurrence_shape"] = "B=1 T=16 Hk=8 Hv=16 Dk=Dv=128, bf16 uniform(-0.1, 0.1), %d input sets in rotation" % nset
+        # the reference's ops fallback at this shape, masked scalar gate, as its C restatement on this box's host cores
+        d0 = {k_: v_.float().cpu().numpy() for k_, v_ in sets[0].items()}
+        cpu = {}
+        for threads in (1, c_oracle.num_threads()):
+            c_oracle.set_num_threads(threads)
+            def med(fn):
+                for _ in range(5):
+                    fn()
+                ts = []
+                for _ in range(20):
+                    t0 = time.perf_counter(); fn(); ts.append(time.perf_counter() - t0)
+                return round(float(np.median(ts)) * 1e6, 1)
+            cpu["threads_%d" % threads] = {
+                "tape_replay_masked_us": med(lambda: c_oracle.tape_replay(d0["tape"], d0["k"], d0["g"], d0["state"], d0["mask"], variant="opbyop")),
+                "gated_delta_masked_us": med(lambda: c_oracle.gated_delta(d0["q"], d0["k"], d0["v"], d0["g"], d0["beta"], d0["state"], d0["mask"],
+                                                                          variant="opbyop"))}
+        out["cpu_ops_fallback_port"] = cpu
+        out["reference_recorded_ops_fallback_us"] = {"tape_replay_masked": 382, "gated_delta_masked": 816,
+                                                     "hardware": "M-series (unspecified)", "source": "DFlashKernels.swift:400-401, :447-448"}
+        Hq, Hkv, D = 32, 8, 128
+        att = {}
+        for nkv in (512, 2048, 8192, 16384, 32768):
+            ns = max(2, min(8, int(600e6 // (Hkv * nkv * D * 4))))
+            asets = [(u(1, Hq, 16, D), u(1, Hkv, nkv, D), u(1, Hkv, nkv, D)) for _ in range(ns)]
+            ws = torch.empty(K.sdpa_workspace_bytes(1, Hq, Hkv, 16, nkv, D), dtype=torch.uint8, device=dev)
+            calls = [(lambda q=q, k=k, v=v: K.batched_sdpa_2pass(q, k, v, D ** -0.5, workspace=ws)) for q, k, v in asets] * max(1, reps // ns)
+            part, comb = timed(_lib.KERNEL_SDPA_PARTIAL, calls), timed(_lib.KERNEL_SDPA_COMBINE, calls)
+            nbytes = (Hq * 16 * D + 2 * Hkv * nkv * D) * 2 + Hq * 16 * D * 2        # the reference's count (main.swift:220-222)
+            att["nKV_%d" % nkv] = {"algorithmic_bytes": nbytes, "sdpa_partial": part, "sdpa_combine": comb,
+                                   "both_us": round(part["median_us"] + comb["median_us"], 2),
+                                   "both_gbs": round(nbytes / (part["median_us"] + comb["median_us"]) / 1e3, 1),
+                                   "both_frac_of_hbm_peak": round(nbytes / (part["median_us"] + comb["median_us"]) / 1e3 / HBM_PEAK_GBS, 4)}
+            del asets, ws
+        out["attention"] = att
+        out["attention_shape"] = "B=1 Hq=32 Hk=8 D=128 bf16, 16 query rows, nKV keys block included"
+    elif name == "config1":
         B, T, Hk, Hv, Dk, Dv, n_layers = 1, 16, 16, 32, 128, 128, 36
         rng = np.random.default_rng(3)
         ns = [int(min(rng.geometric(0.25), T)) for _ in range(n_layers)]
@@ -516,9 +589,10 @@ def main():
     ap.add_argument("--page-size", type=int, default=0,
                     help="keep the attention layers' K/V in paged pools with pages of this many keys (0: dense caches, "
                          "the configuration the headline number is quoted on)")
-    ap.add_argument("--workload", default="config4", choices=["config4", "config1", "config2", "config3"],
+    ap.add_argument("--workload", default="config4", choices=["config4", "config1", "config2", "config3", "refbench"],
                     help="config4 (default) is the benchmark; config1-3 time BASELINE's other configurations at their own "
-                         "shapes (parity-test cases; a separate JSON line, not the headline metric)")
+                         "shapes (parity-test cases; a separate JSON line, not the headline metric); refbench times the shapes "
+                         "and inputs of the reference's own kernel micro-benchmark")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy, the known-size kernel the rocprof byte counters are scaled by")
     args = ap.parse_args()
@@ -654,9 +728,11 @@ def main():
         else:
             one(_lib.KERNEL_TAPE_REPLAY, "tape_replay")
 
+    brk_first = step_no[0]
     for _ in range(brk_steps):
         eager_step(before_launch=arm)
     torch.cuda.synchronize()
+    brk_commits = commits[brk_first:brk_first + brk_steps]
     durs = ev.durations_us()
     avg = lambda key: float(np.mean([durs[i] for i in idx[key]])) if idx[key] else float("nan")
     sdpa_us, comb_us, fwd_us, rep_us = avg("sdpa_partial"), avg("sdpa_combine"), avg("gdn_forward"), avg("tape_replay")
@@ -696,6 +772,25 @@ def main():
 
     mean_commit = int(round(float(np.mean(commits))))
     step_bytes = n_gdn * (stack.gdn_forward_bytes() + stack.replay_bytes(mean_commit)) + n_attn * sdpa_bytes
+    # Every kernel of the step against the HBM peak over its own algorithmic bytes, from the durations of the eager
+    # pass above (events on each dispatch).  "sdpa_pair" is the attention CALL (partial + combine), the unit the
+    # algorithmic bytes are defined for; the replay's bytes are those of the launches that were timed (a fully
+    # accepted step replays nothing and moves nothing).
+    replay_bytes_timed = float(np.mean([n_gdn * stack.replay_bytes(cc) if cc < T else 0 for cc in brk_commits])) if brk_commits else 0.0
+
+    def priced(us, nbytes, launches_per_step):
+        gbs = nbytes / (us * 1e-6) / 1e9
+        return {"avg_launch_us": round(us, 2), "algorithmic_bytes_per_launch": int(nbytes), "gbs": round(gbs, 1),
+                "frac": round(gbs / HBM_PEAK_GBS, 4), "launches_per_step": launches_per_step,
+                "share_of_step": round(us * launches_per_step / (ms_per_step * 1e3), 3)}
+
+    kernels = {
+        "sdpa_partial": priced(sdpa_us, sdpa_bytes, n_attn),
+        "sdpa_pair": priced(sdpa_us + comb_us, sdpa_bytes, n_attn),
+        "gdn_forward_tape": priced(fwd_us, stack.gdn_forward_bytes(), n_gdn),
+        "tape_replay_batched": priced(rep_us, replay_bytes_timed, 1),
+        "unit": "GB/s against the 8000 GB/s HBM peak; durations by HIP events on each dispatch in an eager pass of %d steps" % brk_steps,
+    }
     result = {
         "metric": "dflash_verify_us_per_layer",
         "value": round(us_per_layer, 3),
@@ -734,6 +829,7 @@ def main():
         "step_frac_of_hbm_peak_above_floor": round(step_bytes / ((ms_per_step - floor_us * 1e-3) * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "kernel_us": {"sdpa_partial": round(sdpa_us, 2), "sdpa_combine": round(comb_us, 2),
                       "gdn_forward_tape": round(fwd_us, 2), "tape_replay_batched_36_layers": round(rep_us, 2)},
+        "kernels": kernels,
         "roofline": {
             "kernel": "sdpa_partial_kernel<bf16,256>",
             "bound": "hbm",

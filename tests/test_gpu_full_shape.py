@@ -96,3 +96,45 @@ def test_config4_graph_replay_equals_eager_stepping(gpu_lib):
         assert torch.equal(a["out"], b["out"]) and torch.equal(a["lse"], b["lse"])
         assert torch.equal(a["k_cache"][:, :, :n], b["k_cache"][:, :, :n])
         assert torch.equal(a["v_cache"][:, :, :n], b["v_cache"][:, :, :n])
+
+
+def test_config4_sixty_four_consecutive_steps(gpu_lib):
+    """The benchmark configuration's full run: 64 consecutive verify steps at the full shape, accepted lengths drawn
+    Geometric(0.25) in [1, 16] as the benchmark draws them, stepped the way the benchmark times them (eight steps per
+    captured graph, eight launches).  After the 64th step: cache offset, accept words and the rows every step appended
+    bit-exact; the recurrent state of three GatedDelta layers against the float64 recurrence over exactly the tokens
+    the 64 steps committed (rtol 1e-4); tape, y and the attention outputs of the last step against their restatements."""
+    from bench import StepChecker, draw_commit_counts
+    from swiftlm_amd.verify_step import HybridVerifyStack, StackConfig
+
+    steps, per_graph = 64, 8
+    stack = HybridVerifyStack(StackConfig(max_steps=steps + 2), seed=4, n_slots=per_graph)
+    T = stack.cfg.block
+    commits = draw_commit_counts(steps, T, seed=99)
+    assert 1 in commits and max(commits) > 8
+    commits[5] = T                                           # a fully accepted block (no replay) is part of the run
+    staged, posts = [], []
+    for s, cc in enumerate(commits):
+        stack.set_acceptance(0, cc, seed=s)
+        staged.append(stack.accept_inputs[0].clone())
+        posts.append(stack.posterior[0].cpu())
+    staged = torch.stack(staged)
+    # one eager step on a scratch stack first, so that nothing is set up inside the capture
+    HybridVerifyStack(StackConfig(max_steps=2, n_layers=8), seed=0).enqueue_step()
+    torch.cuda.synchronize()
+    checker = StepChecker(stack, gdn_layers=(0, 17, 35), attn_layers=(0, 11))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        for i in range(per_graph):
+            stack.enqueue_step(slot=i)
+    torch.cuda.current_stream().wait_stream(side)
+    assert stack.phase == 0
+    for r in range(steps // per_graph):
+        stack.accept_inputs[:per_graph].copy_(staged[r * per_graph:(r + 1) * per_graph])
+        g.replay()
+        torch.cuda.synchronize()
+    assert int(stack.offset) == stack.cfg.context + sum(commits)
+    errs = checker.check(commits, posts)
+    assert errs and all(v == v for v in errs.values())

@@ -308,6 +308,20 @@ def test_plain_c_client_of_the_abi(gpu_lib):
     assert "C ABI check passed" in r.stdout
 
 
+def test_plain_c_host_drives_whole_verify_steps_through_a_captured_graph(gpu_lib):
+    """tests/cabi_c/step_check.c: a 3 GatedDelta + 1 attention stack stepped four times by a C99 host through
+    include/dflash_hip.h only -- two steps captured with hipStreamBeginCapture on a fresh stream and launched twice,
+    then the same steps eagerly -- with graph == eager byte for byte and states, offsets, accept words, appended rows
+    and the attention output checked against values computed on the host in C."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "swiftlm_amd", "lib", "step_check")
+    assert os.path.exists(exe), "build it with `make -C swiftlm_amd/csrc`"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "verify-step check passed" in r.stdout
+
+
 # ---- the verify-step driver (what bench.py times): fused and unfused acceptance agree, both match the oracle ----
 
 def test_verify_stack_steps_match_oracle_and_fused_accept(gpu_lib):
