@@ -1294,12 +1294,15 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         //               at that same shared level, hence ordered behind the acknowledged stores);
         //   4. observe  the workgroup whose own increment returns tiles - 1 has observed the increments of all others,
         //               each of which was issued behind that workgroup's acknowledged stores;
-        //   5. acquire  it invalidates what its own caches may hold of those lines (an agent-scope acquire fence: an
-        //               invalidate, not a write-back -- paid by one workgroup per head);
-        //   6. load     and re-reads the head's y and the parked sums (agent-scope loads), finishes the sums, writes `out`.
+        //   5. load     and re-reads the head's y and the parked sums with agent-scope loads, which are served from that
+        //               shared level and never from a copy its own XCD's caches may still hold; then it finishes the
+        //               sums and writes `out`.
         // Steps 1-3 are a release of exactly the lines that are handed over (a release FENCE would also write back the
-        // 2 MB of new state every workgroup has dirtied: 30 us per launch); 4-6 are the matching acquire.  Nothing
-        // waits for anything: a workgroup that is not last is done.
+        // 2 MB of new state every workgroup has dirtied: 30 us per launch); 4-5 are the matching acquire, restricted
+        // to the lines that are read.  An explicit invalidate in front of step 5 (the compiler's agent-scope acquire
+        // fence, or a bare buffer_inv sc1) was measured at +3.4 us per launch (13.2 against 9.8 us) and adds nothing:
+        // the only data that crosses workgroups is read by those agent-scope loads; gate and the norm weight are
+        // inputs of the launch.  Nothing waits for anything: a workgroup that is not last is done.
         if constexpr (FUSED) {
             if (P.fin_gate) {
                 __builtin_amdgcn_s_barrier();       // every wave is past its wait for the y rows (the state stores may be in flight)
@@ -1312,7 +1315,6 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
                 if (arrived >= (int)gridDim.x && P.status && tid == 0) atomicOr(P.status, DFLASH_STATUS_LAYER_ARRIVALS);
                 if (arrived != (int)gridDim.x - 1) return;
                 if (tid == 0) __hip_atomic_store(P.arrivals + bh, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // as the next launch expects it
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
                 if (A.in_dtype == DFLASH_BF16) finish_head(bf16_t{}, tc);
                 else if (A.in_dtype == DFLASH_F16) finish_head(f16_t{}, tc);
                 else finish_head(float{}, tc);
