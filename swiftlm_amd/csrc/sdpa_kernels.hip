@@ -877,20 +877,31 @@ __global__ __launch_bounds__(kCombineThreads) void sdpa_combine_kernel(CombineAr
 static int choose_splits(int B, int Hk, int groups_per_kv, int N) {
     const int nt = (N + kBN - 1) / kBN;
     const int cus = num_compute_units();
-    const int per = B * Hk * groups_per_kv;
-    int S = (cus + per - 1) / per;
-    // Every split pays a fixed price (its partial rows, written once and read back by the combine
-    // kernel, are as large as 4 tiles of K/V), so a short context is not spread thinner than
-    // kMinTilesPerSplit tiles per workgroup.
-    // kMinTilesPerSplit tiles per workgroup, unless that leaves fewer than kMinSplits workgroups
-    // per KV head (then latency, not the partials, is what counts).
-    constexpr int kMinTilesPerSplit = 4, kMinSplits = 32;
-    int floor_s = nt / kMinTilesPerSplit;
-    if (floor_s < kMinSplits) floor_s = kMinSplits;
-    if (S > floor_s) S = floor_s;
+    const int per = B * Hk * groups_per_kv;      // workgroups per split index
+    // How many workgroups W = per * S the key axis is spread over.  Every split pays a fixed price -- its partial rows,
+    // written once and read back by the combine kernel, are as large as 4 tiles of K/V, and a launch drains them all at
+    // once -- while a workgroup streams a tile in about 1.2 us.  Measured on split counts swept at 4K .. 100K keys
+    // (Hq=16, Hk=2, D=256; microseconds for the pair of launches):
+    //     keys     W=64   W=128   W=172   W=256
+    //     4112     14.0   13.6      -     16.0          8208     17.8   15.7    -     17.6
+    //     16400    19.8   20.6   19.8     20.9          32784      -    28.8   26.7   25.9
+    // i.e. half the chip up to about two tiles per compute unit, the whole chip from eight tiles per compute unit on,
+    // linear in between; never more workgroups than tiles.
+    const long total_tiles = (long)per * nt;
+    long W = cus / 2 + (total_tiles - 2L * cus) / 12;
+    if (W < cus / 2) W = cus / 2;
+    if (W > cus) W = cus;
+    int S = (int)((W + per - 1) / per);
     if (S > nt) S = nt;
     if (S > kMaxSplits) S = kMaxSplits;
     if (S < 1) S = 1;
+    // If a few more splits (at most a quarter, and never more workgroups than compute units) take one tile off the
+    // longest split, take them: 129 tiles over 64 splits leave one split with three, over 65 splits none.
+    const int longest = (nt + S - 1) / S;
+    if (longest > 1) {
+        const int more = (nt + longest - 2) / (longest - 1);          // splits for a longest one of longest - 1 tiles
+        if (more <= S + S / 4 && (long)more * per <= cus && more <= kMaxSplits) S = more;
+    }
     return S;
 }
 
