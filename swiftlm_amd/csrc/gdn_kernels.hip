@@ -457,6 +457,7 @@ __global__ __launch_bounds__(kThreads) void gated_delta_tape_kernel(GdnArgs A) {
     constexpr int ROWS = kThreads / LPR;
     constexpr int CH = DK / (4 * LPR);
     constexpr int TC = kGdnChunk;
+    constexpr int TPR = DK / 4;                                   // threads spanning one step's q (or k) row, 4 channels each
     static_assert(CH >= 1, "row slice must hold at least one float4");
 
     __shared__ float q_s[TC][DK];
@@ -466,9 +467,11 @@ __global__ __launch_bounds__(kThreads) void gated_delta_tape_kernel(GdnArgs A) {
     __shared__ float y_s[TC][ROWS];
     __shared__ float t_s[TC][ROWS];
     __shared__ float beta_s[TC];
-    __shared__ float kq_s[TC];
     __shared__ int on_s[TC];
 
+    // every argument in one burst of scalar loads (fetched where first used they are several dependent trips to memory)
+    asm volatile("" ::"s"(A.q), "s"(A.k), "s"(A.v), "s"(A.g), "s"(A.beta), "s"(A.mask), "s"(A.state_in), "s"(A.state_out),
+                 "s"(A.y), "s"(A.tape), "s"(A.in_dtype), "s"(A.mask_dtype), "s"(A.T), "s"(A.Hk), "s"(A.Hv), "s"(A.Dv));
     const int bh = blockIdx.y;
     const int b = bh / A.Hv, hv = bh % A.Hv;
     const int hk = hv / (A.Hv / A.Hk);
@@ -482,9 +485,97 @@ __global__ __launch_bounds__(kThreads) void gated_delta_tape_kernel(GdnArgs A) {
     const StateT* s_in = reinterpret_cast<const StateT*>(A.state_in) + ((size_t)bh * A.Dv + (row_ok ? row : 0)) * DK;
     StateT* s_out = reinterpret_cast<StateT*>(A.state_out) + ((size_t)bh * A.Dv + (row_ok ? row : 0)) * DK;
 
+    // The state rows are the largest operand: their loads go out first.
     float4 s[CH];
 #pragma unroll
     for (int c = 0; c < CH; ++c) s[c] = load4(s_in + c * 4 * LPR + 4 * j);
+
+    // ---- a chunk's operands: requested as raw bits, array by array, inside branches that hold nothing but loads, and
+    // converted only after the last request has gone out -- one memory round trip per chunk.  (With a conversion or an
+    // LDS store next to each load, or a switch on the element type around it, the compiler waits for every load before
+    // it issues the next: half a dozen dependent round trips per launch.)  Addresses are clamped instead of predicated;
+    // values that must not count are dropped at the LDS store. ----
+    constexpr int QI = (TC * TPR + kThreads - 1) / kThreads;      // q / k (and vector gate) groups of 4 per thread
+    constexpr int VI = (TC * ROWS + kThreads - 1) / kThreads;     // v values per thread
+    const bool in32 = A.in_dtype == DFLASH_F32, in_bf16 = A.in_dtype == DFLASH_BF16;
+    uint4 q32[QI], k32[QI], g32[VEC_G ? QI : 1];
+    uint2 q16[QI], k16[QI], g16[VEC_G ? QI : 1];
+    float v32[VI], gs32 = 1.f, bs32 = 0.f;
+    uint32_t v16[VI], gs16 = 0, bs16 = 0;                         // 16-bit values, zero-extended
+    int on_r = 1;
+    auto cvt16 = [](uint16_t bits, bool is_bf16) -> float {
+        return is_bf16 ? __uint_as_float(((uint32_t)bits) << 16) : (float)__builtin_bit_cast(_Float16, bits);
+    };
+    auto cvt4 = [&](uint4 w, uint2 h) -> float4 {
+        if (in32) return make_float4(__uint_as_float(w.x), __uint_as_float(w.y), __uint_as_float(w.z), __uint_as_float(w.w));
+        return make_float4(cvt16((uint16_t)(h.x & 0xffffu), in_bf16), cvt16((uint16_t)(h.x >> 16), in_bf16),
+                           cvt16((uint16_t)(h.y & 0xffffu), in_bf16), cvt16((uint16_t)(h.y >> 16), in_bf16));
+    };
+    auto request_chunk = [&](int t0, int tc) {
+        size_t kidx[QI], gidx[QI], vidx[VI];
+#pragma unroll
+        for (int u = 0; u < QI; ++u) {
+            const int i = tid + u * kThreads, c = (i % TPR) * 4;
+            const int t = (i / TPR) < tc ? (i / TPR) : tc - 1;
+            const size_t bt = (size_t)b * A.T + t0 + t;
+            kidx[u] = (bt * A.Hk + hk) * DK + c;
+            gidx[u] = (bt * A.Hv + hv) * DK + c;
+        }
+#pragma unroll
+        for (int u = 0; u < VI; ++u) {
+            const int i = tid + u * kThreads, r = i % ROWS;
+            const int t = (i / ROWS) < tc ? (i / ROWS) : tc - 1;
+            const int rr = (row0 + r) < A.Dv ? row0 + r : A.Dv - 1;
+            vidx[u] = (((size_t)b * A.T + t0 + t) * A.Hv + hv) * A.Dv + rr;
+        }
+        const int tl = tid < tc ? tid : tc - 1;
+        const size_t bts = (size_t)b * A.T + t0 + tl;
+        if (in32) {
+#pragma unroll
+            for (int u = 0; u < QI; ++u) {
+                q32[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const float*>(A.q) + kidx[u]);
+                k32[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const float*>(A.k) + kidx[u]);
+                if (VEC_G) g32[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const float*>(A.g) + gidx[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < VI; ++u) v32[u] = reinterpret_cast<const float*>(A.v)[vidx[u]];
+            if (!VEC_G) gs32 = reinterpret_cast<const float*>(A.g)[bts * A.Hv + hv];
+            bs32 = reinterpret_cast<const float*>(A.beta)[bts * A.Hv + hv];
+        } else {
+#pragma unroll
+            for (int u = 0; u < QI; ++u) {
+                q16[u] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(A.q) + kidx[u]);
+                k16[u] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(A.k) + kidx[u]);
+                if (VEC_G) g16[u] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(A.g) + gidx[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < VI; ++u) v16[u] = reinterpret_cast<const uint16_t*>(A.v)[vidx[u]];
+            if (!VEC_G) gs16 = reinterpret_cast<const uint16_t*>(A.g)[bts * A.Hv + hv];
+            bs16 = reinterpret_cast<const uint16_t*>(A.beta)[bts * A.Hv + hv];
+        }
+        if (HAS_MASK) on_r = (int)mask_on(A.mask, A.mask_dtype, (int)bts);
+    };
+    auto park_chunk = [&](int tc) {
+#pragma unroll
+        for (int u = 0; u < QI; ++u) {
+            const int i = tid + u * kThreads, t = i / TPR, c = (i % TPR) * 4;
+            if (t < tc) {
+                store4(&q_s[t][c], cvt4(q32[u], q16[u]));
+                store4(&k_s[t][c], cvt4(k32[u], k16[u]));
+                if (VEC_G) store4(&g_s[t][c], cvt4(g32[VEC_G ? u : 0], g16[VEC_G ? u : 0]));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < VI; ++u) {
+            const int i = tid + u * kThreads, t = i / ROWS, r = i % ROWS;
+            if (t < tc) v_s[t][r] = (row0 + r) < A.Dv ? (in32 ? v32[u] : cvt16((uint16_t)v16[u], in_bf16)) : 0.f;
+        }
+        if (tid < tc) {
+            if (!VEC_G) g_s[0][tid] = in32 ? gs32 : cvt16((uint16_t)gs16, in_bf16);
+            beta_s[tid] = in32 ? bs32 : cvt16((uint16_t)bs16, in_bf16);
+            if (HAS_MASK) on_s[tid] = on_r;
+        }
+    };
 
     auto fetch = [&](int t, GdnStepOps<CH>& o) {
 #pragma unroll
@@ -497,41 +588,26 @@ __global__ __launch_bounds__(kThreads) void gated_delta_tape_kernel(GdnArgs A) {
         o.gs = VEC_G ? 1.f : g_s[0][t];
         o.v = v_s[t][rloc];
         o.beta = beta_s[t];
-        o.kq = kq_s[t];
         o.on = HAS_MASK ? on_s[t] : 1;
+        // k.q of the step (one value per head and step) from the lane's own channels; it does not depend on the
+        // state, so its reduction runs beside the step-to-step chain, not on it
+        float kq0 = 0.f, kq1 = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            kq0 = fmaf(o.k[c].x, o.q[c].x, kq0); kq1 = fmaf(o.k[c].y, o.q[c].y, kq1);
+            kq0 = fmaf(o.k[c].z, o.q[c].z, kq0); kq1 = fmaf(o.k[c].w, o.q[c].w, kq1);
+        }
+        o.kq = group_sum<LPR>(kq0 + kq1);
     };
 
+    if (A.T > 0) request_chunk(0, A.T < TC ? A.T : TC);
     for (int t0 = 0; t0 < A.T; t0 += TC) {
         const int tc = (A.T - t0) < TC ? (A.T - t0) : TC;
-        if (t0) __syncthreads();
-        // ---- stage operands of this chunk as float ----
-        for (int i = tid; i < tc * (DK / 4); i += kThreads) {
-            const int t = i / (DK / 4), c = (i % (DK / 4)) * 4;
-            const size_t bt = (size_t)b * A.T + t0 + t;
-            store4(&q_s[t][c], load4_rt(A.q, A.in_dtype, (bt * A.Hk + hk) * DK + c));
-            store4(&k_s[t][c], load4_rt(A.k, A.in_dtype, (bt * A.Hk + hk) * DK + c));
-            if (VEC_G) store4(&g_s[t][c], load4_rt(A.g, A.in_dtype, (bt * A.Hv + hv) * DK + c));
+        if (t0) {
+            __syncthreads();                      // every wave is done with the previous chunk's operands and outputs
+            request_chunk(t0, tc);
         }
-        for (int i = tid; i < tc * ROWS; i += kThreads) {
-            const int t = i / ROWS, r = i % ROWS;
-            const size_t bt = (size_t)b * A.T + t0 + t;
-            v_s[t][r] = (row0 + r) < A.Dv ? load1_rt(A.v, A.in_dtype, (bt * A.Hv + hv) * A.Dv + row0 + r) : 0.f;
-        }
-        if (tid < tc) {
-            const size_t bt = (size_t)b * A.T + t0 + tid;
-            if (!VEC_G) g_s[0][tid] = load1_rt(A.g, A.in_dtype, bt * A.Hv + hv);
-            beta_s[tid] = load1_rt(A.beta, A.in_dtype, bt * A.Hv + hv);
-            if (HAS_MASK) on_s[tid] = (int)mask_on(A.mask, A.mask_dtype, (int)bt);
-        }
-        __syncthreads();
-
-        // k.q per step (one value per head and step): 16 lanes per step
-        for (int t = tid / 16; t < tc; t += kThreads / 16) {
-            float acc = 0.f;
-            for (int d = tid % 16; d < DK; d += 16) acc = fmaf(k_s[t][d], q_s[t][d], acc);
-            acc = group_sum<16>(acc);
-            if (tid % 16 == 0) kq_s[t] = acc;
-        }
+        park_chunk(tc);
         __syncthreads();
 
         // ---- serial steps, operands one step ahead (two operand sets, no register copies) ----
@@ -564,14 +640,28 @@ __global__ __launch_bounds__(kThreads) void gated_delta_tape_kernel(GdnArgs A) {
             }
             if (j == 0) { y_s[t][rloc] = yv; t_s[t][rloc] = delta; }
         };
-        GdnStepOps<CH> opa, opb;
-        fetch(0, opa);
-        for (int t = 0; t < tc; t += 2) {
-            if (t + 1 < tc) fetch(t + 1, opb);
-            step(t, opa);
-            if (t + 1 < tc) {
-                if (t + 2 < tc) fetch(t + 2, opa);
-                step(t + 1, opb);
+        if (tc == TC) {
+            // A full chunk (the verify block) is straight-line code: operands are fetched kAhead steps ahead of their
+            // use, so no step waits for LDS.
+            constexpr int kAhead = 4;
+            GdnStepOps<CH> ops[TC];
+#pragma unroll
+            for (int t = 0; t < kAhead; ++t) fetch(t, ops[t]);
+#pragma unroll
+            for (int t = 0; t < TC; ++t) {
+                if (t + kAhead < TC) fetch(t + kAhead, ops[t + kAhead]);
+                step(t, ops[t]);
+            }
+        } else {
+            GdnStepOps<CH> opa, opb;
+            fetch(0, opa);
+            for (int t = 0; t < tc; t += 2) {
+                if (t + 1 < tc) fetch(t + 1, opb);
+                step(t, opa);
+                if (t + 1 < tc) {
+                    if (t + 2 < tc) fetch(t + 2, opa);
+                    step(t + 1, opb);
+                }
             }
         }
         __syncthreads();
