@@ -336,7 +336,22 @@ def aux_kernels(lib, cfg, reps=48):
         out[label] = {"us": round(us, 2), "algorithmic_bytes": nbytes, "gbs": round(nbytes / us / 1e3, 1),
                       "kernel": "chunked (MFMA)" if sb == 4 else "serial (state re-rounded per step)"}
         ev.destroy()
-    del qs
+    # What a launch costs that only moves the recurrent state of one layer (read 2 MiB, write 2 MiB) with the forward's
+    # own decomposition over the chip: the tape replay of zero steps is exactly that copy.  The floor under the
+    # GatedDelta forward's launch: everything the forward adds to it is its arithmetic and its small operands.
+    copies = [(s_, torch.empty_like(s_)) for *_, s_ in qs]
+    zero_t = [(q_[:, :0].contiguous(), k_[:, :0].contiguous(), g_[:, :0].contiguous()) for q_, k_, _, g_, _, _ in qs]
+    ev = HipEvents()
+    for (s_in, _), (_, k0, g0) in zip(copies, zero_t):
+        e0, e1 = ev.pair()
+        _lib.check(lib.dflash_profile_next_launch(_lib.KERNEL_TAPE_REPLAY, e0, e1), "profile_next_launch")
+        K.tape_replay_kernel(torch.empty(B, 0, Hv, Dv, device=dev), k0, g0, s_in)
+    torch.cuda.synchronize()
+    us = float(np.median(ev.durations_us()))
+    out["state_copy_floor"] = {"us": round(us, 2), "bytes": 2 * Hv * Dv * Dk * 4, "gbs": round(2 * Hv * Dv * Dk * 4 / us / 1e3, 1),
+                               "what": "tape replay of zero steps: one layer's fp32 state read and written, nothing else"}
+    ev.destroy()
+    del qs, copies
 
     V = 151936
     logits = [torch.randn(T, V, generator=g, device=dev).to(bf) for _ in range(reps)]      # 48 x 4.9 MB
