@@ -797,10 +797,9 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
                      "s"(P.q_scale), "s"(P.k_scale), "s"(P.eps), "s"(P.C));
     if constexpr (FUSED)
         asm volatile("" ::"s"(P.fin_gate), "s"(P.fin_weight), "s"(P.fin_out), "s"(P.arrivals), "s"(P.status), "s"(P.fin_eps), "s"(P.fin_silu));
-    if constexpr (!FUSED)
-        asm volatile("" ::"s"(A.q), "s"(A.k), "s"(A.v), "s"(A.g), "s"(A.beta), "s"(A.mask), "s"(A.state_in), "s"(A.state_out),
-                     "s"(A.y), "s"(A.tape), "s"(A.in_dtype), "s"(A.mask_dtype), "s"(A.T), "s"(A.Hk), "s"(A.Hv), "s"(A.Dv),
-                     "s"(A.group), "s"(A.group_magic));
+    // (The plain forward gets what its first loads need -- the state pointer, k, q and the sizes in their addresses -- in
+    //  SGPRs at wave start, as leading kernel arguments; the rest of its arguments are named in one such statement
+    //  further down, behind those loads, so that the wait for the argument block does not stand in front of them.)
     constexpr int E = DK / 64;             // channels per lane in the state-update product (16 lanes x E x 4 waves = DK)
     static_assert(DK % 64 == 0, "chunked gated delta needs Dk to be a multiple of 64");
 
@@ -810,10 +809,10 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
     // q/k/v/g/beta/y/tape are 32-bit (the host checks the sizes), their per-thread parts 24-bit multiplies.
     const int b = blockIdx.z, hv = blockIdx.y;
     const int bh = b * A.Hv + hv;
-    const int hk = A.group == 1 ? hv : (int)__umulhi((uint32_t)hv, A.group_magic);
+    const int hk = A.group == 1 ? hv : (FUSED ? (int)__umulhi((uint32_t)hv, A.group_magic) : (int)((uint32_t)hv / A.group));
     const int row0 = blockIdx.x * kChunkRows;
     const float* s_in = reinterpret_cast<const float*>(A.state_in) + ((size_t)bh * A.Dv + row0) * DK;
-    float* s_out = reinterpret_cast<float*>(A.state_out) + ((size_t)bh * A.Dv + row0) * DK;
+    const size_t tile_off = ((size_t)bh * A.Dv + row0) * DK;          // of this workgroup's rows in the state arrays
     const uint32_t k_step = (uint32_t)A.Hk * DK, v_step = (uint32_t)A.Hv * A.Dv;       // elements per step
 
     constexpr int NV = kChunkRows * (DK / 4) / kThreads;      // float4 groups per thread of a 16 x DK tile
@@ -823,7 +822,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
             const int i = tid + u * kThreads, r = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
-            store4(s_out + (size_t)r * DK + c4, load4(s_in + (size_t)r * DK + c4));
+            store4(reinterpret_cast<float*>(A.state_out) + tile_off + (size_t)r * DK + c4, load4(s_in + (size_t)r * DK + c4));
         }
         return;
     }
@@ -900,6 +899,11 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
             on = HAS_MASK ? mask_on(A.mask, A.mask_dtype, (int)(bt0 + tl)) : true;
             on = on && tid < tc;
         }
+        // The arguments that were not handed over in registers, in one burst of scalar loads, behind every load of the
+        // chunk (pinned: the scheduler would otherwise lift the first use of one of them, and with it the wait for the
+        // argument block, in front of the loads).
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("" ::"s"(A.mask), "s"(A.state_out), "s"(A.y), "s"(A.tape), "s"(A.in_dtype), "s"(A.mask_dtype));
         if (with_state) {
 #pragma unroll
             for (int u = 0; u < NV; ++u) {
@@ -1345,6 +1349,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
                 for (int e = 0; e < E; ++e)
                     cacc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, L.y[s][base + e], cacc[e], 0, 0, 0);
             }
+            float* const s_out = reinterpret_cast<float*>(A.state_out) + tile_off;      // first use of the pointer: down here
             if (last_chunk) {
                 // (layer kernel with the gated norm inside: the wave's y rows and sums of squares must be acknowledged
                 //  before it counts itself in; waited for here, ahead of the state stores, the wait does not include
@@ -1416,8 +1421,18 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         for (int t0 = kChunkSteps; t0 < A.T; t0 += kChunkSteps) run_chunk(t0);
 }
 
+// What stands between a wave's start and its loads -- the six input pointers and the sizes their addresses need --
+// is passed as leading scalar arguments: the command processor hands those over in SGPRs when the wave starts (kernarg
+// preload, 14 dwords at most, hence the sizes packed in pairs), so no load waits for a trip to the argument block.
+// The rest of the arguments (outputs, mask, types) follow in the struct and are fetched while the loads are in flight.
 template <bool HAS_MASK, int DK, bool BF>
-__global__ __launch_bounds__(kThreads) void gated_delta_chunk_kernel(GdnArgs A) {
+__global__ __launch_bounds__(kThreads) void gated_delta_chunk_kernel(const void* state_in, const void* k, const void* q, const void* v,
+                                                                     const void* g, const void* beta, uint32_t hv_dv, uint32_t hk_t,
+                                                                     GdnArgs A) {
+    A.state_in = state_in; A.k = k; A.q = q; A.v = v; A.g = g; A.beta = beta;
+    A.Hv = (int)(hv_dv >> 16); A.Dv = (int)(hv_dv & 0xffffu); A.Hk = (int)(hk_t >> 16); A.T = (int)(hk_t & 0xffffu);
+    A.group = (uint32_t)A.Hv / (uint32_t)A.Hk;
+    A.group_magic = 0;                 // hk = hv / group is divided out below (scalar, once): the reciprocal did not fit the registers
     gdn_chunk_body<HAS_MASK, DK, false, BF>(A, GdnPrep{});
 }
 
@@ -1455,10 +1470,11 @@ static int launch_gdn_chunk(hipStream_t st, const GdnArgs& A, int B) {
     dim3 grid(A.Dv / kChunkRows, A.Hv, B);
     LaunchBracket br(DFLASH_KERNEL_GDN_FORWARD, st);
     const bool bf = A.in_dtype == DFLASH_BF16;
-    if (A.mask && bf) br.launch(gated_delta_chunk_kernel<true, DK, true>, grid, dim3(kThreads), lds, A);
-    else if (A.mask) br.launch(gated_delta_chunk_kernel<true, DK, false>, grid, dim3(kThreads), lds, A);
-    else if (bf) br.launch(gated_delta_chunk_kernel<false, DK, true>, grid, dim3(kThreads), lds, A);
-    else br.launch(gated_delta_chunk_kernel<false, DK, false>, grid, dim3(kThreads), lds, A);
+    const uint32_t hv_dv = ((uint32_t)A.Hv << 16) | (uint32_t)A.Dv, hk_t = ((uint32_t)A.Hk << 16) | (uint32_t)A.T;   // each below 2^16, checked by the caller
+    if (A.mask && bf) br.launch(gated_delta_chunk_kernel<true, DK, true>, grid, dim3(kThreads), lds, A.state_in, A.k, A.q, A.v, A.g, A.beta, hv_dv, hk_t, A);
+    else if (A.mask) br.launch(gated_delta_chunk_kernel<true, DK, false>, grid, dim3(kThreads), lds, A.state_in, A.k, A.q, A.v, A.g, A.beta, hv_dv, hk_t, A);
+    else if (bf) br.launch(gated_delta_chunk_kernel<false, DK, true>, grid, dim3(kThreads), lds, A.state_in, A.k, A.q, A.v, A.g, A.beta, hv_dv, hk_t, A);
+    else br.launch(gated_delta_chunk_kernel<false, DK, false>, grid, dim3(kThreads), lds, A.state_in, A.k, A.q, A.v, A.g, A.beta, hv_dv, hk_t, A);
     DFLASH_HIP_TRY(hipGetLastError());
     return DFLASH_OK;
 }
@@ -1575,7 +1591,7 @@ extern "C" int dflash_gated_delta_tape(void* stream, const void* q, const void* 
     A.q = q; A.k = k; A.v = v; A.g = g; A.beta = beta; A.mask = mask;
     A.state_in = state_in; A.state_out = state_out; A.y = y; A.tape = tape_out;
     A.in_dtype = in_dtype; A.mask_dtype = mask_dtype; A.T = T; A.Hk = Hk; A.Hv = Hv; A.Dv = Dv;
-    if (state_dtype == DFLASH_F32 && g_ndim == 3 && Dv % kChunkRows == 0 && T > 0 && chunk_index_setup(A, B, Dk)) {
+    if (state_dtype == DFLASH_F32 && g_ndim == 3 && Dv % kChunkRows == 0 && T > 0 && T < 65536 && Dv < 65536 && chunk_index_setup(A, B, Dk)) {
         // fp32 state with one decay per head and step: chunked form
         if (Dk == 64) return launch_gdn_chunk<64>((hipStream_t)stream, A, B);
         if (Dk == 128) return launch_gdn_chunk<128>((hipStream_t)stream, A, B);
