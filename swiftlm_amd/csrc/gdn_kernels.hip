@@ -1405,8 +1405,8 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
         //   5. load     and re-reads the head's y and the parked sums with agent-scope loads, which are served from that
         //               shared level and never from a copy its own XCD's caches may still hold; then it finishes the
         //               sums and writes `out`.
-        // Steps 1-3 are a release of exactly the lines that are handed over (a release FENCE would also write back the
-        // 2 MB of new state every workgroup has dirtied: 30 us per launch); 4-5 are the matching acquire, restricted
+        // Steps 1-3 are a release of exactly the lines that are handed over (a release FENCE is a write-back of the whole
+        // L2: 30 us per launch when it was tried, with the new state still stored write-back); 4-5 are the matching acquire, restricted
         // to the lines that are read.  An explicit invalidate in front of step 5 (the compiler's agent-scope acquire
         // fence, or a bare buffer_inv sc1) was measured at +3.4 us per launch (13.2 against 9.8 us) and adds nothing:
         // the only data that crosses workgroups is read by those agent-scope loads; gate and the norm weight are
