@@ -601,6 +601,10 @@ def main():
     ap.add_argument("--aux", action="store_true",
                     help="also time the kernels next to the measured path (pre-ops, greedy tokens) and report them "
                          "under aux_kernels; they are not part of the step time")
+    ap.add_argument("--no-post-block-state", action="store_true",
+                    help="variant, not the headline: the GatedDelta forwards do not store the state after the whole block "
+                         "(state_out = NULL) and the rollback replays the tape also when every token is accepted; the "
+                         "reference's forward returns that state, so this is not the drop-in call sequence")
     ap.add_argument("--page-size", type=int, default=0,
                     help="keep the attention layers' K/V in paged pools with pages of this many keys (0: dense caches, "
                          "the configuration the headline number is quoted on)")
@@ -635,6 +639,7 @@ def main():
     G = max(2, args.steps_per_graph & ~1)
     cfg = StackConfig(context=args.context, max_steps=total + 2, page_size=args.page_size)
     stack = HybridVerifyStack(cfg, seed=0, n_slots=G)
+    stack.post_block_state = not args.no_post_block_state
     T = cfg.block
     commits = draw_commit_counts(total, T)
     # token ids of every step, staged on the device once
@@ -826,6 +831,8 @@ def main():
             "layers": cfg.n_layers, "block": T, "context": cfg.context,
             "launch": "eager" if graphs is None else "hip-graph, %d steps per graph" % G,
             "kv_layout": "dense" if not cfg.page_size else "paged, %d-key pages" % cfg.page_size,
+            "gdn_post_block_state": "stored by every forward (the reference's call sequence)" if stack.post_block_state
+                                    else "NOT stored; the rollback replays whole blocks too (variant, not the drop-in sequence)",
         },
         "verified": True,
         "verified_how": ("two further steps run like the timed ones, then on the live buffers: offsets and accept words and "

@@ -110,6 +110,14 @@ int dflash_tape_replay_batched(void* stream, int n_layers,
  *   q,k,v,g,beta : in_dtype          y : in_dtype        tape_out : float32
  *   state        : state_dtype (F32, or == in_dtype with per-step re-rounding,
  *                  DFlashKernels.swift:183-186)
+ * state_out may be NULL: the post-block state is then not stored.  It is only
+ * ever read when a block is accepted whole (DFlashRuntime.swift:194-202 keeps it
+ * then; every other outcome replays from the snapshot and overwrites it), so a
+ * host that rolls back with dflash_tape_replay* whatever was accepted
+ * (skip_if_full = 0) does not need it, and the launch is about a tenth shorter
+ * without the store.  Only the form used for verify blocks supports this (fp32
+ * state, g_ndim == 3, Dk in {64,128,256}, Dv % 16 == 0, T >= 1); other shapes
+ * return DFLASH_UNSUPPORTED when state_out is NULL.
  * ---------------------------------------------------------------------- */
 int dflash_gated_delta_tape(void* stream,
                             const void* q, const void* k, const void* v,

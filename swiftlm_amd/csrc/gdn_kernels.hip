@@ -820,6 +820,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
     const int ts = tid / 16, tt = tid % 16;        // (s, t) for the tables, (t, r) for v / y / tape
 
     if (A.T == 0) {                        // nothing to do but hand the state over
+        if (A.state_out == nullptr) return;
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
             const int i = tid + u * kThreads, r = i / (DK / 4), c4 = (i % (DK / 4)) * 4;
@@ -1359,6 +1360,8 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
                     if (P.fin_gate) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 // Written through (system scope) like y and the tape: the 2 MB of new state then drain while the launch
                 // still runs instead of waiting dirty in the L2s for the end-of-launch flush (-0.7 % of a verify step).
+                // A caller that rolls back from the tape whatever is accepted passes no state_out: nothing is stored.
+                if (A.state_out != nullptr)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     float* const ptr = s_out + (uint32_t)((4 * kk + v) * DK + base);
@@ -1592,7 +1595,7 @@ extern "C" int dflash_gated_delta_tape(void* stream, const void* q, const void* 
     DFLASH_REQUIRE(B > 0 && T >= 0 && Hk > 0 && Hv > 0 && Dk > 0 && Dv > 0, "gated delta: non-positive dimension");
     DFLASH_REQUIRE(Hv % Hk == 0, "gated delta: Hv=%d is not a multiple of Hk=%d", Hv, Hk);
     DFLASH_REQUIRE(g_ndim == 3 || g_ndim == 4, "gated delta: g_ndim must be 3 or 4");
-    DFLASH_REQUIRE(state_in && state_out, "gated delta: null state pointer");
+    DFLASH_REQUIRE(state_in, "gated delta: null state pointer");
     DFLASH_REQUIRE(state_in != state_out, "gated delta: state_in aliases state_out");
     DFLASH_REQUIRE(T == 0 || (q && k && v && g && beta && y && tape_out), "gated delta: null pointer");
     DFLASH_REQUIRE((long)B * Hv <= 65535, "gated delta: B*Hv too large for one launch");
@@ -1610,6 +1613,8 @@ extern "C" int dflash_gated_delta_tape(void* stream, const void* q, const void* 
         if (Dk == 128) return launch_gdn_chunk<128>((hipStream_t)stream, A, B);
         if (Dk == 256) return launch_gdn_chunk<256>((hipStream_t)stream, A, B);
     }
+    DFLASH_SUPPORTED(state_out != nullptr, "gated delta: a call without state_out needs the chunked form (fp32 state, one decay "
+                     "per head and step, Dk in {64, 128, 256}, Dv a multiple of 16, T >= 1)");
     switch (state_dtype) {
         case DFLASH_F32: return launch_gdn_state<float>((hipStream_t)stream, A, B, g_ndim, Dk);
         case DFLASH_BF16: return launch_gdn_state<bf16_t>((hipStream_t)stream, A, B, g_ndim, Dk);

@@ -110,12 +110,14 @@ class DFlashKernels:
     @staticmethod
     def gated_delta_kernel_with_tape(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor,
                                      beta: torch.Tensor, state: torch.Tensor,
-                                     mask: Optional[torch.Tensor] = None
-                                     ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+                                     mask: Optional[torch.Tensor] = None, want_state: bool = True
+                                     ) -> Tuple[torch.Tensor, Optional[torch.Tensor], torch.Tensor]:
         """``gatedDeltaKernelWithTape(q:k:v:g:beta:state:mask:)`` (DFlashKernels.swift:316-367).
 
         Returns (y [B,T,Hv,Dv] in q's dtype, new state in ``state``'s dtype,
-        innovation tape [B,T,Hv,Dv] float32)."""
+        innovation tape [B,T,Hv,Dv] float32).  ``want_state=False`` (no counterpart in the reference) leaves the
+        post-block state out -- None is returned in its place -- for a caller that replays the tape whatever is
+        accepted; only the verify-block form supports it (``DFlashUnsupported`` otherwise)."""
         _dev(q, k, v, g, beta, state, mask)
         q, k, v, g, beta, state = (t.contiguous() for t in (q, k, v, g, beta, state))
         for name, t in (("k", k), ("v", v), ("g", g), ("beta", beta)):
@@ -126,7 +128,7 @@ class DFlashKernels:
         Hv, Dv = v.shape[2], v.shape[3]
         y = torch.empty((B, T, Hv, Dv), dtype=q.dtype, device=q.device)
         tape = torch.empty((B, T, Hv, Dv), dtype=torch.float32, device=q.device)
-        out = torch.empty_like(state)
+        out = torch.empty_like(state) if want_state else None
         rc = _lib.load().dflash_gated_delta_tape(
             _stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(g), g.dim(), _ptr(beta), _code(q),
             _ptr(state), _ptr(out), _code(state), _ptr(y), _ptr(tape),

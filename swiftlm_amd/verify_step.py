@@ -68,6 +68,10 @@ class HybridVerifyStack:
         self.cfg = cfg
         self.lib = _lib.load()
         self.fuse_accept = True      # acceptance decided inside the batched replay launch (one launch fewer per step)
+        # False: the forwards do not store the post-block state and the rollback replays the tape also when the whole
+        # block is accepted (no counterpart in the reference, whose forward returns that state; the committed state
+        # is the same either way)
+        self.post_block_state = True
         g = torch.Generator(device=device).manual_seed(seed)
         bf = torch.bfloat16
         T = cfg.block
@@ -156,8 +160,8 @@ class HybridVerifyStack:
                 note("gdn_forward")
                 rc = lib.dflash_gated_delta_tape(
                     st, _p(l["q"]), _p(l["k"]), _p(l["v"]), _p(l["g"]), 3, _p(l["beta"]), _lib.BF16,
-                    _p(l["state"][ph]), _p(l["state"][1 - ph]), _lib.F32, _p(l["y"]), _p(l["tape"]), None, 0,
-                    1, T, cfg.Hk, cfg.Hv, cfg.Dk, cfg.Dv)
+                    _p(l["state"][ph]), _p(l["state"][1 - ph]) if self.post_block_state else None, _lib.F32, _p(l["y"]),
+                    _p(l["tape"]), None, 0, 1, T, cfg.Hk, cfg.Hv, cfg.Dk, cfg.Dv)
                 _lib.check(rc, "gated_delta_tape")
             else:
                 l = self.attn[ai]; ai += 1
@@ -186,7 +190,8 @@ class HybridVerifyStack:
             rc = lib.dflash_accept_commit_replay_batched(
                 st, _p(self.verify_ids[slot]), _p(self.posterior[slot]), T, _p(self.offset), _p(self.accept),
                 len(self.gdn), cast(tb["tape"]), _lib.F32, cast(tb["k"]), cast(tb["g"]), _lib.BF16, 3,
-                cast(tb["sin"]), cast(tb["sout"]), _lib.F32, 1, 1, T, cfg.Hk, cfg.Hv, cfg.Dk, cfg.Dv)
+                cast(tb["sin"]), cast(tb["sout"]), _lib.F32, 1 if self.post_block_state else 0, 1, T, cfg.Hk, cfg.Hv,
+                cfg.Dk, cfg.Dv)
             _lib.check(rc, "accept_commit_replay_batched")
             self.phase = 1 - ph
             return
@@ -200,8 +205,8 @@ class HybridVerifyStack:
             note("tape_replay")
             rc = lib.dflash_tape_replay_batched(
                 st, len(self.gdn), cast(tb["tape"]), _lib.F32, cast(tb["k"]), cast(tb["g"]), _lib.BF16, 3,
-                cast(tb["sin"]), cast(tb["sout"]), _lib.F32, 0, C.c_void_p(self.accept.data_ptr() + 4), 1,
-                1, T, cfg.Hk, cfg.Hv, cfg.Dk, cfg.Dv)
+                cast(tb["sin"]), cast(tb["sout"]), _lib.F32, 0, C.c_void_p(self.accept.data_ptr() + 4),
+                1 if self.post_block_state else 0, 1, T, cfg.Hk, cfg.Hv, cfg.Dk, cfg.Dv)
             _lib.check(rc, "tape_replay_batched")
         self.phase = 1 - ph
 

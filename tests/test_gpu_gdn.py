@@ -223,6 +223,33 @@ def test_batched_replay_equals_per_layer_replay(gpu_lib):
     assert all(bool((m == 7.0).all()) for m in marker)
 
 
+@pytest.mark.parametrize("shape", [("cfg1", 1, 16, 16, 32, 128, 128), ("cfg0", 1, 8, 4, 8, 64, 64), ("dk256", 1, 6, 1, 2, 256, 64),
+                                   ("long_T", 1, 40, 2, 4, 64, 32)], ids=lambda s: s[0])
+@pytest.mark.parametrize("in_dt", ["f32", "bf16"])
+def test_forward_without_post_block_state(gpu_lib, shape, in_dt):
+    """state_out = NULL: y and the tape are the bits of the ordinary call, no state is written anywhere, and replaying
+    the whole tape from the same start gives the state the ordinary call returns (to the state's bar)."""
+    from swiftlm_amd import DFlashKernels as K, DFlashUnsupported
+
+    _, B, T, Hk, Hv, Dk, Dv = shape
+    d = O.make_gdn_inputs(77, B, T, Hk, Hv, Dk, Dv, in_dtype=in_dt)
+    q, k, v, g, beta = (dev(d[n], in_dt) for n in ("q", "k", "v", "g", "beta"))
+    s0 = dev(d["state"])
+    keep = s0.clone()
+    y1, s1, t1 = K.gated_delta_kernel_with_tape(q, k, v, g, beta, s0)
+    y2, s2, t2 = K.gated_delta_kernel_with_tape(q, k, v, g, beta, s0, want_state=False)
+    torch.cuda.synchronize()
+    assert s2 is None
+    assert torch.equal(y1, y2) and torch.equal(t1, t2)
+    assert torch.equal(s0, keep)
+    rep = K.tape_replay_kernel(t2, k, g, s0)
+    np.testing.assert_allclose(host(rep), host(s1), **STATE_TOL)
+    # the step-by-step kernel (per-channel gate, low-precision state) always stores its state
+    dv = O.make_gdn_inputs(78, 1, 4, 2, 4, 64, 16, vec_gate=True)
+    with pytest.raises(DFlashUnsupported):
+        K.gated_delta_kernel_with_tape(*(dev(dv[n]) for n in ("q", "k", "v", "g", "beta")), dev(dv["state"]), want_state=False)
+
+
 def test_unsupported_and_invalid_arguments(gpu_lib):
     from swiftlm_amd import DFlashKernels as K, DFlashError, DFlashUnsupported
 

@@ -365,6 +365,45 @@ def test_verify_stack_steps_match_oracle_and_fused_accept(gpu_lib):
             np.testing.assert_allclose(host(la["out"]), ow, rtol=2e-2, atol=2e-2)
 
 
+def test_verify_stack_without_post_block_state_commits_the_same_states(gpu_lib):
+    """The variant in which no forward stores the state after the whole block and the rollback replays the tape also
+    for a block accepted whole: bookkeeping and attention identical; tapes, y and committed states identical bit for
+    bit until a block is accepted whole (the same replay from the same tape), and to the state's bar from then on (that
+    block's state is a replay of 16 steps instead of the forward's own state, and the later steps start from it)."""
+    import torch
+    from swiftlm_amd.verify_step import HybridVerifyStack, StackConfig
+
+    cfg = StackConfig(n_layers=8, attn_every=4, block=16, Hk=2, Hv=4, Dk=128, Dv=32, Hq=4, Hkv=2, D=128,
+                      context=150, max_steps=6)
+    for fuse in (True, False):
+        a, b = HybridVerifyStack(cfg, seed=3), HybridVerifyStack(cfg, seed=3)
+        a.fuse_accept = b.fuse_accept = fuse
+        b.post_block_state = False
+        same_bits = True
+        for step, cc in enumerate([3, 16, 1, 16, 9]):
+            for st in (a, b):
+                st.set_acceptance(st.phase, cc, seed=step)
+                if st is b:                                  # nothing may rely on what the buffer held before
+                    for l in st.gdn:
+                        l["state"][1 - st.phase].fill_(float("nan"))
+                st.enqueue_step()
+            torch.cuda.synchronize()
+            assert a.accept.tolist() == b.accept.tolist() and int(a.offset) == int(b.offset)
+            for la, lb in zip(a.gdn, b.gdn):
+                sa, sb = la["state"][a.phase], lb["state"][b.phase]
+                assert bool(torch.isfinite(sb).all())
+                if same_bits:
+                    assert torch.equal(la["tape"], lb["tape"]) and torch.equal(la["y"], lb["y"])
+                    if cc < cfg.block:
+                        assert torch.equal(sa, sb)
+                np.testing.assert_allclose(host(lb["tape"]), host(la["tape"]), rtol=1e-4, atol=1e-5)
+                np.testing.assert_allclose(host(lb["y"]), host(la["y"]), rtol=2e-2, atol=2e-2)
+                np.testing.assert_allclose(host(sb), host(sa), rtol=1e-4, atol=1e-5)
+            same_bits = same_bits and cc < cfg.block
+            for la, lb in zip(a.attn, b.attn):
+                assert torch.equal(la["out"], lb["out"]) and torch.equal(la["lse"], lb["lse"])
+
+
 def test_verify_stack_paged_equals_dense(gpu_lib):
     """The verify-step driver with paged K/V pools gives the bytes of the dense driver, step after step,
     and the appended rows sit in the pages the table names."""
