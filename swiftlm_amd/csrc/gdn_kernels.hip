@@ -1351,7 +1351,8 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
                 for (int e = 0; e < E; ++e)
                     cacc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, L.y[s][base + e], cacc[e], 0, 0, 0);
             }
-            float* const s_out = reinterpret_cast<float*>(A.state_out) + tile_off;      // first use of the pointer: down here
+            // first use of the pointer: down here (null when the caller does not want the post-block state)
+            float* const s_out = A.state_out ? reinterpret_cast<float*>(A.state_out) + tile_off : nullptr;
             if (last_chunk) {
                 // (layer kernel with the gated norm inside: the wave's y rows and sums of squares must be acknowledged
                 //  before it counts itself in; waited for here, ahead of the state stores, the wait does not include
@@ -1361,7 +1362,7 @@ __device__ __forceinline__ void gdn_chunk_body(const GdnArgs& A, const GdnPrep& 
                 // Written through (system scope) like y and the tape: the 2 MB of new state then drain while the launch
                 // still runs instead of waiting dirty in the L2s for the end-of-launch flush (-0.7 % of a verify step).
                 // A caller that rolls back from the tape whatever is accepted passes no state_out: nothing is stored.
-                if (A.state_out != nullptr)
+                if (s_out != nullptr)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     float* const ptr = s_out + (uint32_t)((4 * kk + v) * DK + base);
