@@ -193,3 +193,14 @@ def test_argument_validation_needs_no_gpu_for_null_checks():
     assert lib.dflash_cache_rollback(None, None, 0) == _lib.INVALID
     assert lib.dflash_cache_set_slot(None, 0, None) == _lib.INVALID
     assert lib.dflash_restore_target_cache_after_acceptance(None, 3, None, 0, 0, 0, None) == _lib.INVALID
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it says so and exits non-zero without touching a device."""
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stdout + r.stderr)
